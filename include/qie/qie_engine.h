@@ -266,7 +266,7 @@ int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_id
  * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains; each branch is
  * normed after it is computed, its input is the raw stream); the next layer's input is the depth-weighted sum over the embedding
  * output and every layer result so far. */
-enum { QIE_MIXER_LATENT_ATTENTION = 1, QIE_MIXER_GQA = 2, QIE_MIXER_GQA_RECURRENT = 3 };
+enum { QIE_MIXER_LATENT_ATTENTION = 1, QIE_MIXER_GQA = 2, QIE_MIXER_GQA_RECURRENT = 3, QIE_MIXER_MINGRU = 4 };
 enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
 /* Which keys j <= i a query at position i sees: all of them; the last `size`; those of its own
  * block of `size` positions (blocks counted from position 0 of the sequence). */
@@ -278,11 +278,27 @@ enum { QIE_QKNORM_NONE = 0, QIE_QKNORM_WEIGHT = 1, QIE_QKNORM_PLAIN = 2 };
 enum { QIE_ROT_HALVES = 0, QIE_ROT_INTERLEAVED = 1 };
 /* Block: 0 = y = x + g * rms(branch(x)) with scalar gains (branches read the raw stream);
  * 1 = x += N_b(branch(N_a(x))) with weight vectors stored around zero (N(v) = rms(v) (1 + w))
- * before and after every branch. */
-enum { QIE_BLOCK_POSTNORM_GAIN = 0, QIE_BLOCK_SANDWICH = 1 };
+ * before and after every branch; 2 = x += branch(N(x)) with N(v) = rms(v) w (plain weight vectors
+ * 'l<i>.norm1|norm2', 'final.norm'), one norm before every branch and none after. */
+enum { QIE_BLOCK_POSTNORM_GAIN = 0, QIE_BLOCK_SANDWICH = 1, QIE_BLOCK_PRENORM = 2 };
 /* Router: 0 = sigmoid scores, the `top` largest scale the experts' input; 1 = logits with a
  * bias, the `top` largest weighted by the softmax over those alone scale the experts' output. */
-enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1 };
+enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1, QIE_ROUTER_SOFTMAX_ALL = 2 };
+/* Router 2: scores s = softmax over ALL router outputs (`experts` experts with weights, then
+ * `identity` experts whose output is their input); experts are chosen by s + correction ('l<i>.mlp.
+ * correction'), only inside the `groups_keep` best of `groups` equal groups of neighbouring
+ * outputs (a group's rank: its largest s + correction); the `top` chosen are weighted by
+ * s / (sum of the chosen s + 1e-20) * route_scale, applied to the experts' outputs. */
+/* Dense feed-forward: 0 = W_down (silu(W_gate h) * W_up h); 1 = W_down xielu(W_up h) with the two
+ * numbers p, q of 'l<i>.mlp.act': xielu(z) = softplus(p) z^2 + z / 2 for z > 0, else
+ * (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.  Experts are always of form 0. */
+enum { QIE_ACT_SILU_GATED = 0, QIE_ACT_XIELU = 1 };
+/* Attention weights of the visible keys: softmax of the scores, or sigmoid(score + pb_h) with a
+ * number per head ('mix.pb'), not normalised over the keys. */
+enum { QIE_WEIGHTS_SOFTMAX = 0, QIE_WEIGHTS_SIGMOID = 1 };
+/* Positions in the embedding: none, or the vector with entry 2i = sin(p * 10000^(-2i / width)),
+ * entry 2i + 1 = cos of the same, added to the scaled embedding row. */
+enum { QIE_POS_NONE = 0, QIE_POS_SINUSOID = 1 };
 
 /* Mixer QIE_MIXER_GQA: grouped-query softmax attention over a paged K / V cache.  q = W_q h
  * (heads x dim), k = W_k h (kv_heads x dim), v = W_v h (kv_heads x vdim); query head h reads
@@ -303,6 +319,12 @@ typedef struct qie_gqa_desc {
     int32_t dist_bias;
     float rot_base, scale;
     int32_t reserved[2];
+    int32_t weights;          /* QIE_WEIGHTS_*                                               */
+    int32_t slope_bias;       /* 1: the score loses 2^(-8 (h + 1) / heads) * (i - j)         */
+    int32_t head_gate;        /* 1: head h's output times sigmoid(W_g x)_h ('mix.g' [heads, width]) */
+    int32_t q_temp_every;     /* > 0: after its norm q is multiplied by                      */
+    float q_temp_coef;        /*   1 + coef * ln(floor((pos + 1) / every) + 1)               */
+    int32_t reserved2[3];
 } qie_gqa_desc;
 
 /* Gated linear recurrence (the second half of QIE_MIXER_GQA_RECURRENT): per head a state
@@ -315,6 +337,16 @@ typedef struct qie_recurrent_desc {
     int32_t heads, dim, vdim;
     int32_t reserved;
 } qie_recurrent_desc;
+
+/* Mixer QIE_MIXER_MINGRU: a gated recurrence whose gates read only the current token.  With x the
+ * mixer's input: z = sigmoid(W_z x + b_z), u = W_x x + b_x (`width` channels each), candidate
+ * c = u + 1/2 where u >= 0, sigmoid(u) where u < 0; per channel S_t = (1 - z_t) S_(t-1) + z_t c_t,
+ * S fp32 in the slot, zero at position 0; output W_o (S_t * silu(W_g x)).  Tensors
+ * 'l<i>.mix.z|z.b|x|x.b|g|o'. */
+typedef struct qie_mingru_desc {
+    int32_t width;
+    int32_t reserved[3];
+} qie_mingru_desc;
 
 typedef struct qie_layer_desc {
     int32_t mixer;            /* QIE_MIXER_*                                          */
@@ -331,6 +363,12 @@ typedef struct qie_layer_desc {
     qie_gqa_desc gqa;         /* QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT                */
     qie_recurrent_desc rec;   /* QIE_MIXER_GQA_RECURRENT                               */
     float gqa_scale, rec_scale;
+    qie_mingru_desc mingru;   /* QIE_MIXER_MINGRU                                      */
+    int32_t ff_act;           /* QIE_ACT_* of a dense feed-forward                     */
+    int32_t identity;         /* QIE_ROUTER_SOFTMAX_ALL: identity experts after the `experts` real ones */
+    int32_t groups, groups_keep;
+    float route_scale;
+    int32_t reserved3[3];
 } qie_layer_desc;
 
 typedef struct qie_arch_desc {
@@ -343,7 +381,8 @@ typedef struct qie_arch_desc {
      * run with its own cache region and state); before every run of the group but the first
      * the embedding rows are added to the stream.  loop_times <= 1: every layer once. */
     int32_t loop_start, loop_stop, loop_times;
-    int32_t reserved[2];
+    int32_t pos_embed;        /* QIE_POS_*                                              */
+    float embed_scale;        /* the embedding row is multiplied by it (0 is read as 1) */
     const qie_layer_desc* layers;
 } qie_arch_desc;
 
@@ -353,7 +392,8 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
  * 'l<i>.norm1b|norm2b', all vectors of the width), 'l<i>.mix.q|dkv|dkv.norm|uk|uv|g|o' (latent
  * attention), 'l<i>.mix.q|k|v|q.norm|k.norm|r1|r2|o' (QIE_MIXER_GQA; under 'l<i>.mix.left.' when a
  * recurrence runs beside it, whose tensors are 'l<i>.mix.right.q|f|f.b|lower|v|norm|o'),
- * 'l<i>.mlp.gate|up|down|router|router.b', 'l<i>.mlp.e<j>.gate|up|down'.
+ * 'l<i>.mix.pb|g' (sigmoid weights, head gate), 'l<i>.mix.z|z.b|x|x.b|g|o' (QIE_MIXER_MINGRU),
+ * 'l<i>.mlp.gate|up|down|act|router|router.b|correction', 'l<i>.mlp.e<j>.gate|up|down'.
  * qie_engine_finalize_weights checks every tensor the architecture needs against its shape,
  * builds the device layouts (fused projection rows, per-head transposed W_uk, experts end to
  * end) and drops the host copies. */
@@ -386,8 +426,8 @@ int qie_batch_keep_layers(qie_batch* b, int32_t enable);
 int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n);
 /* Time `iters` runs of one stage of the last step's shape (hipEvents on the engine stream):
  * which 0 = the whole layer stack, 1 = attention of `layer`, 2 = its projections (input, absorb,
- * value expansion, output), 3 = its feed-forward, 4 = its gated recurrence (scan + head norm; the
- * slots' states of that layer run are advanced by it, so time it last).  The cache is read, not
+ * value expansion, output), 3 = its feed-forward, 4 = its recurrence (gated scan + head norm, or the
+ * minGRU scan; the slots' states of that layer run are advanced by it, so time it last).  The cache is read, not
  * advanced. */
 int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us);
 

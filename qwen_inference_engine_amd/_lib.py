@@ -81,24 +81,33 @@ class EngineOptsC(C.Structure):
                 ("compute_f32", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
-QIE_MIXER_LATENT_ATTENTION, QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT = 1, 2, 3
+QIE_MIXER_LATENT_ATTENTION, QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT, QIE_MIXER_MINGRU = 1, 2, 3, 4
 QIE_FF_NONE, QIE_FF_DENSE, QIE_FF_MOE = 0, 1, 2
 QIE_MASK_CAUSAL, QIE_MASK_WINDOW, QIE_MASK_CHUNK = 0, 1, 2
 QIE_QKNORM_NONE, QIE_QKNORM_WEIGHT, QIE_QKNORM_PLAIN = 0, 1, 2
 QIE_ROT_HALVES, QIE_ROT_INTERLEAVED = 0, 1
-QIE_BLOCK_POSTNORM_GAIN, QIE_BLOCK_SANDWICH = 0, 1
-QIE_ROUTER_SIGMOID_IN, QIE_ROUTER_SOFTMAX_OUT = 0, 1
+QIE_BLOCK_POSTNORM_GAIN, QIE_BLOCK_SANDWICH, QIE_BLOCK_PRENORM = 0, 1, 2
+QIE_ROUTER_SIGMOID_IN, QIE_ROUTER_SOFTMAX_OUT, QIE_ROUTER_SOFTMAX_ALL = 0, 1, 2
+QIE_ACT_SILU_GATED, QIE_ACT_XIELU = 0, 1
+QIE_WEIGHTS_SOFTMAX, QIE_WEIGHTS_SIGMOID = 0, 1
+QIE_POS_NONE, QIE_POS_SINUSOID = 0, 1
 
 
 class GqaDescC(C.Structure):
     _fields_ = [("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32),
                 ("qk_norm", C.c_int32), ("rot_dims", C.c_int32), ("rot_layout", C.c_int32), ("rot_values", C.c_int32),
                 ("mask", C.c_int32), ("mask_size", C.c_int32), ("values_are_keys", C.c_int32), ("dist_bias", C.c_int32),
-                ("rot_base", C.c_float), ("scale", C.c_float), ("reserved", C.c_int32 * 2)]
+                ("rot_base", C.c_float), ("scale", C.c_float), ("reserved", C.c_int32 * 2),
+                ("weights", C.c_int32), ("slope_bias", C.c_int32), ("head_gate", C.c_int32), ("q_temp_every", C.c_int32),
+                ("q_temp_coef", C.c_float), ("reserved2", C.c_int32 * 3)]
 
 
 class RecurrentDescC(C.Structure):
     _fields_ = [("heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32), ("reserved", C.c_int32)]
+
+
+class MinGruDescC(C.Structure):
+    _fields_ = [("width", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
 class LayerDescC(C.Structure):
@@ -107,14 +116,16 @@ class LayerDescC(C.Structure):
                 ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("scale", C.c_float),
                 ("ff_kind", C.c_int32), ("ff", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
                 ("router", C.c_int32), ("reserved", C.c_int32 * 3),
-                ("gqa", GqaDescC), ("rec", RecurrentDescC), ("gqa_scale", C.c_float), ("rec_scale", C.c_float)]
+                ("gqa", GqaDescC), ("rec", RecurrentDescC), ("gqa_scale", C.c_float), ("rec_scale", C.c_float),
+                ("mingru", MinGruDescC), ("ff_act", C.c_int32), ("identity", C.c_int32), ("groups", C.c_int32),
+                ("groups_keep", C.c_int32), ("route_scale", C.c_float), ("reserved3", C.c_int32 * 3)]
 
 
 class ArchDescC(C.Structure):
     _fields_ = [("n_layers", C.c_int32), ("width", C.c_int32), ("vocab", C.c_int32), ("norm_eps", C.c_float),
                 ("depth_mix", C.c_int32), ("block", C.c_int32), ("tied_head", C.c_int32),
                 ("loop_start", C.c_int32), ("loop_stop", C.c_int32), ("loop_times", C.c_int32),
-                ("reserved", C.c_int32 * 2), ("layers", C.POINTER(LayerDescC))]
+                ("pos_embed", C.c_int32), ("embed_scale", C.c_float), ("layers", C.POINTER(LayerDescC))]
 
 
 # (name, restype, argtypes) — every symbol the public headers declare.

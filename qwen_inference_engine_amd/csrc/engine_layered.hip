@@ -62,9 +62,18 @@ struct LayerDev {
     int rope_v = 0;
     float *qn_w = nullptr, *kn_w = nullptr, *r1 = nullptr, *r2 = nullptr;
     float *rec_fb = nullptr, *rec_lower = nullptr, *rec_norm = nullptr;
-    // sandwich blocks: weight vectors of the four norms; biased routers
+    // sandwich blocks: weight vectors of the four norms (pre-norm blocks: n1, n2); biased routers
     float *n1 = nullptr, *n1b = nullptr, *n2 = nullptr, *n2b = nullptr;
     float* router_b = nullptr;
+    // attention options: head slopes of the linear distance bias, the sigmoid weights' bias per head,
+    // the column of the head gates inside the fused projection (-1: none)
+    float *slopes = nullptr, *pb = nullptr;
+    int col_gate = -1;
+    // QIE_MIXER_MINGRU: w_in = [z ; x ; g] rows, wo = W_o; biases of z and x
+    float *mg_zb = nullptr, *mg_xb = nullptr;
+    // xIELU: softplus(p), 1/2 + softplus(q); the grouped router's correction
+    float act_p = 0.f, act_q = 0.f;
+    float* correction = nullptr;
 };
 
 // One execution of a layer: layers of a repeated group run several times, each run with its
@@ -84,7 +93,8 @@ struct LayeredModel {
     void* embed = nullptr;
     void* head = nullptr;
     float g_final = 1.f;
-    float* w_final = nullptr;   // sandwich blocks: the output norm's weight vector
+    float* w_final = nullptr;   // sandwich and pre-norm blocks: the output norm's weight vector
+    double* pos_freq = nullptr; // sinusoidal positions: 10000^(-2i / width), i < ceil(width / 2)
     std::vector<LayerRun> runs;
     bool loops = false;
     std::vector<void*> allocs;
@@ -290,7 +300,9 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
     const int64_t rq = rec ? (int64_t)d.rec.heads * d.rec.dim : 0, rv = rec ? (int64_t)d.rec.heads * d.rec.vdim : 0;
     L.col_k = (int)nq;
     L.col_v = a.values_are_keys ? -1 : (int)(nq + nk);
-    L.col_rq = (int)(nq + nk + nv);
+    const int64_t ng = a.head_gate ? a.heads : 0;
+    L.col_gate = a.head_gate ? (int)(nq + nk + nv) : -1;
+    L.col_rq = (int)(nq + nk + nv + ng);
     L.col_rf = (int)(L.col_rq + rq);
     L.col_rv = (int)(L.col_rf + rq);
     L.n_in = (int)(L.col_rv + rv);
@@ -310,6 +322,19 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
     if (a.dist_bias) {
         QIE_TRY(lm_vector(m, &L.r1, pa + "r1", a.heads));
         QIE_TRY(lm_vector(m, &L.r2, pa + "r2", a.heads));
+    }
+    if (a.head_gate) {
+        LM_GET(tg, pa + "g", (int64_t)a.heads, W);
+        QIE_TRY(lm_upload_rows(m, L.w_in, L.col_gate, W, *tg));
+    }
+    if (a.weights == QIE_WEIGHTS_SIGMOID) QIE_TRY(lm_vector(m, &L.pb, pa + "pb", a.heads));
+    if (a.slope_bias) {
+        HostTensor sl;
+        sl.dtype = 2;
+        sl.shape = {(int64_t)a.heads};
+        sl.data.resize((size_t)a.heads * 4);
+        for (int h = 0; h < a.heads; h++) ((float*)sl.data.data())[h] = (float)std::exp2(-8.0 * (h + 1) / a.heads);
+        QIE_TRY(lm_floats(m, &L.slopes, sl));
     }
     if (a.rot_dims > 0) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.rot_dims, &L.rope));
     if (a.rot_values) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.vdim, &L.rope_v));
@@ -349,6 +374,28 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
 
 static int finalize_ff(LayeredModel* m, int i);
 
+// minGRU: fused input rows [z ; x ; g], the two bias vectors, W_o
+static int finalize_mingru(LayeredModel* m, int i) {
+    LayerDev& L = m->L[i];
+    const int64_t W = m->a.width, n = L.d.mingru.width;
+    const std::string px = "l" + std::to_string(i) + ".mix.";
+    L.n_in = (int)(3 * n);
+    L.n_cat = (int)n;
+    QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
+    LM_GET(tz, px + "z", n, W);
+    LM_GET(tx, px + "x", n, W);
+    LM_GET(tg, px + "g", n, W);
+    QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tz));
+    QIE_TRY(lm_upload_rows(m, L.w_in, n, W, *tx));
+    QIE_TRY(lm_upload_rows(m, L.w_in, 2 * n, W, *tg));
+    QIE_TRY(lm_vector(m, &L.mg_zb, px + "z.b", n));
+    QIE_TRY(lm_vector(m, &L.mg_xb, px + "x.b", n));
+    LM_GET(to, px + "o", W, n);
+    QIE_TRY(lm_alloc(m, &L.wo, (size_t)W * n * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.wo, 0, n, *to));
+    return 0;
+}
+
 static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
     LayerDev& L = m->L[i];
     const qie_layer_desc& d = L.d;
@@ -361,6 +408,14 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
             QIE_TRY(lm_vector(m, &L.n2, pl + "norm2", Wn));
             QIE_TRY(lm_vector(m, &L.n2b, pl + "norm2b", Wn));
         }
+    }
+    if (m->a.block == QIE_BLOCK_PRENORM) {
+        QIE_TRY(lm_vector(m, &L.n1, pl + "norm1", m->a.width));
+        if (d.ff_kind != QIE_FF_NONE) QIE_TRY(lm_vector(m, &L.n2, pl + "norm2", m->a.width));
+    }
+    if (d.mixer == QIE_MIXER_MINGRU) {
+        QIE_TRY(finalize_mingru(m, i));
+        return finalize_ff(m, i);
     }
     if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
         QIE_TRY(finalize_gqa_mixer(e, m, i));
@@ -420,7 +475,18 @@ static int finalize_ff(LayeredModel* m, int i) {
     const int64_t W = m->a.width;
     const std::string pl = "l" + std::to_string(i) + ".";
     const int64_t ff = d.ff;
-    if (d.ff_kind == QIE_FF_DENSE) {
+    if (d.ff_kind == QIE_FF_DENSE && d.ff_act == QIE_ACT_XIELU) {
+        LM_GET(wu, pl + "mlp.up", ff, W);
+        LM_GET(wd, pl + "mlp.down", W, ff);
+        LM_GET(wa, pl + "mlp.act", (int64_t)2);
+        QIE_TRY(lm_alloc(m, &L.w_gu, (size_t)ff * W * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_gu, 0, W, *wu));
+        QIE_TRY(lm_alloc(m, &L.w_down, (size_t)W * ff * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_down, 0, ff, *wd));
+        auto softplus = [](double z) { return std::log1p(std::exp(-std::fabs(z))) + std::max(z, 0.0); };
+        L.act_p = (float)softplus((double)host_elem(*wa, 0));
+        L.act_q = (float)(0.5 + softplus((double)host_elem(*wa, 1)));
+    } else if (d.ff_kind == QIE_FF_DENSE) {
         LM_GET(wg, pl + "mlp.gate", ff, W);
         LM_GET(wu, pl + "mlp.up", ff, W);
         LM_GET(wd, pl + "mlp.down", W, ff);
@@ -430,11 +496,12 @@ static int finalize_ff(LayeredModel* m, int i) {
         QIE_TRY(lm_alloc(m, &L.w_down, (size_t)W * ff * m->esz()));
         QIE_TRY(lm_upload_rows(m, L.w_down, 0, ff, *wd));
     } else if (d.ff_kind == QIE_FF_MOE) {
-        const int64_t E = d.experts;
-        LM_GET(wr, pl + "mlp.router", E, W);
-        QIE_TRY(lm_alloc(m, &L.w_router, (size_t)E * W * m->esz()));
+        const int64_t E = d.experts, ER = E + (d.router == QIE_ROUTER_SOFTMAX_ALL ? d.identity : 0);
+        LM_GET(wr, pl + "mlp.router", ER, W);
+        QIE_TRY(lm_alloc(m, &L.w_router, (size_t)ER * W * m->esz()));
         QIE_TRY(lm_upload_rows(m, L.w_router, 0, W, *wr));
         if (d.router == QIE_ROUTER_SOFTMAX_OUT) QIE_TRY(lm_vector(m, &L.router_b, pl + "mlp.router.b", E));
+        if (d.router == QIE_ROUTER_SOFTMAX_ALL) QIE_TRY(lm_vector(m, &L.correction, pl + "mlp.correction", ER));
         QIE_TRY(lm_alloc(m, &L.w_gu, (size_t)E * 2 * ff * W * m->esz()));
         QIE_TRY(lm_alloc(m, &L.w_down, (size_t)E * W * ff * m->esz()));
         for (int64_t x = 0; x < E; x++) {
@@ -661,17 +728,30 @@ static int enq_ff(qie_batch* b, int i, int T) {
     LayeredBatch* s = b->lb;
     const int W = m->a.width, ff = d.ff;
     hipStream_t st = e->stream;
+    if (d.ff_kind == QIE_FF_DENSE && d.ff_act == QIE_ACT_XIELU) {
+        QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, ff, T, ff, W, s->y_bf));
+        QIE_TRY(lay::xielu(s->gu, s->act, s->act_bf, (int64_t)T * ff, L.act_p, L.act_q, st));
+        return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff, s->act_bf);
+    }
     if (d.ff_kind == QIE_FF_DENSE) {
         QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, 2 * ff, T, 2 * ff, W, s->y_bf));
         QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, T, ff, st));
         return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff, s->act_bf);
     }
     const int E = d.experts, top = d.top, n = T * top;
-    const bool out_w = d.router == QIE_ROUTER_SOFTMAX_OUT;   // the scores weight the outputs, not the inputs
+    const bool out_w = d.router != QIE_ROUTER_SIGMOID_IN;   // the scores weight the outputs, not the inputs
     const float* in_score = out_w ? nullptr : s->score;
     const float* out_score = out_w ? s->score : nullptr;
-    QIE_TRY(lay::route_topk(s->y, L.w_router, L.router_b, m->f32, T, W, E, top, out_w ? 1 : 0, s->sel, s->score, st));
-    QIE_TRY(lay::moe_group(s->sel, n, E, s->cnt, s->off, s->slot_of, st));
+    // identity experts follow the real ones in the router's outputs: they get groups of their own in
+    // the row order below, no products, and the combine takes the rows' input for them
+    const int ER = E + (d.router == QIE_ROUTER_SOFTMAX_ALL ? d.identity : 0);
+    const int32_t* id_sel = ER > E ? s->sel : nullptr;
+    if (d.router == QIE_ROUTER_SOFTMAX_ALL)
+        QIE_TRY(lay::route_grouped(s->y, L.w_router, L.correction, m->f32, T, W, ER, top, d.groups, d.groups_keep, d.route_scale,
+                                   s->sel, s->score, st));
+    else
+        QIE_TRY(lay::route_topk(s->y, L.w_router, L.router_b, m->f32, T, W, E, top, out_w ? 1 : 0, s->sel, s->score, st));
+    QIE_TRY(lay::moe_group(s->sel, n, ER, s->cnt, s->off, s->slot_of, st));
     const bool per_expert = !m->f32 && n >= kMoeSyncRows && W % 8 == 0 && ff % 8 == 0;
     QIE_TRY(lay::moe_gather(s->y, in_score, s->slot_of, T, top, W, s->xg, per_expert ? s->xg_bf : nullptr, st));
     if (per_expert) {
@@ -714,12 +794,12 @@ static int enq_ff(qie_batch* b, int i, int T) {
                                  lane_of(x)));
         }
         QIE_TRY(join());
-        return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st);
+        return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st, id_sel, E, s->y);
     }
     QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
     QIE_TRY(lay::silu_mul(s->gu, s->act, nullptr, n, ff, st));
     QIE_TRY(lin(e, s->act, ff, L.w_down, ff, s->yd, W, n, W, ff, E, 0, (int64_t)W * ff, 0, s->off));
-    return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st);
+    return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st, id_sel, E, s->y);
 }
 
 // ---- grouped-query attention (+ gated recurrence) of layer run r; the branch input is s->y
@@ -746,6 +826,9 @@ static lay::GqaAttnP gqa_attn_params(qie_batch* b, int r) {
     p.v_transposed = s->v_transposed;
     p.out_scale = L.d.mixer == QIE_MIXER_GQA_RECURRENT ? L.d.gqa_scale : 1.0f;
     p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = L.n_cat; p.out_col = 0;
+    p.slopes = a.slope_bias ? L.slopes : nullptr;
+    p.pb = a.weights == QIE_WEIGHTS_SIGMOID ? L.pb : nullptr;
+    p.gate_col = a.head_gate ? L.col_gate : -1;
     return p;
 }
 
@@ -781,6 +864,8 @@ static int enq_gqa_post(qie_batch* b, int r, int T) {
     p.k_off = s->layer_off[r];
     p.v_off = s->v_off[r];
     p.v_transposed = s->v_transposed;
+    p.q_temp_every = a.q_temp_every;
+    p.q_temp_coef = a.q_temp_coef;
     return lay::gqa_post(p, m->f32, T, e->stream);
 }
 
@@ -869,6 +954,83 @@ static int enq_gqa_mixer(qie_batch* b, int r, int T) {
     return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
 }
 
+// minGRU of layer run r: the scan over the fused projection rows -> s->ov (gated, with its bf16 image).
+// Entries above kScanLong rows run in pieces: piece-local end states and decay products from zero
+// states, a carry pass over each entry's pieces, then the pieces again from the states that enter
+// them (the same recurrence, regrouped: S_end = decay * S_in + S_local).
+static int enq_mingru(qie_batch* b, int r, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    const int n = L.d.mingru.width;
+    lay::MinGruScanP p{};
+    p.proj = s->proj; p.ld = L.n_in; p.z_col = 0; p.x_col = n; p.g_col = 2 * n;
+    p.z_b = L.mg_zb; p.x_b = L.mg_xb;
+    p.n = n;
+    p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = n;
+    if (s->max_count > kScanLong && s->s_loc) {
+        lay::MinGruScanP a = p;
+        a.entries = s->d_chunks; a.n_entries = s->n_chunks;
+        a.out = nullptr; a.out_bf = nullptr;
+        a.end = s->s_loc; a.decay = s->s_decay; a.end_stride = n; a.end_off = 0;
+        QIE_TRY(lay::mingru_scan(a, e->stream));
+        lay::MinGruCarryP k{s->d_spans, s->n_ent, n, s->s_loc, s->s_decay, s->s_in, s->state, s->slot_state, s->state_off[r]};
+        QIE_TRY(lay::mingru_carry(k, e->stream));
+        a = p;
+        a.entries = s->d_chunks; a.n_entries = s->n_chunks;
+        a.init = s->s_in; a.init_stride = n; a.init_off = 0; a.init_if_pos = 0;
+        return lay::mingru_scan(a, e->stream);
+    }
+    p.entries = s->d_ent; p.n_entries = s->n_ent;
+    p.init = s->state; p.init_stride = s->slot_state; p.init_off = s->state_off[r]; p.init_if_pos = 1;
+    p.end = s->state; p.end_stride = s->slot_state; p.end_off = s->state_off[r];
+    return lay::mingru_scan(p, e->stream);
+}
+
+static int enq_mingru_mixer(qie_batch* b, int r, int T) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    QIE_TRY(dense(b, s->y, m->a.width, L.w_in, s->proj, L.n_in, T, L.n_in, m->a.width, s->y_bf));
+    QIE_TRY(enq_mingru(b, r, T));
+    return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
+}
+
+// Pre-norm blocks: x += mixer(N1(x)); x += ff(N2(x)), plain weight vectors.  The stream lives in
+// plane 1 of the stack; every residual add is fused with the norm that reads its result (the last
+// kernel of a run makes the next run's input unless the streams are kept).
+static int enq_run_prenorm(qie_batch* b, int r, int T, bool h_ready, bool* next_ready) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    hipStream_t st = e->stream;
+    float* x = s->stack + s->cap * W;
+    const float eps = m->a.norm_eps;
+    if (!h_ready) QIE_TRY(lay::add_norm(x, x, nullptr, nullptr, nullptr, L.n1, s->y, s->y_bf, T, W, eps, st, 0.f));
+    if (L.d.mixer == QIE_MIXER_MINGRU)
+        QIE_TRY(enq_mingru_mixer(b, r, T));
+    else
+        QIE_TRY(enq_gqa_mixer(b, r, T));
+    const bool has_ff = L.d.ff_kind != QIE_FF_NONE;
+    const bool last = r + 1 == (int)m->runs.size();
+    const bool fuse_next = !last && !s->keep_on;
+    const float* next_w = fuse_next ? m->L[m->runs[r + 1].layer].n1 : nullptr;
+    if (has_ff) {
+        QIE_TRY(lay::add_norm(x, x, s->mix, nullptr, nullptr, L.n2, s->y, s->y_bf, T, W, eps, st, 0.f));
+        QIE_TRY(enq_ff(b, m->runs[r].layer, T));
+        QIE_TRY(lay::add_norm(x, x, s->ffo, nullptr, nullptr, next_w, s->y, s->y_bf, T, W, eps, st, 0.f));
+    } else {
+        QIE_TRY(lay::add_norm(x, x, s->mix, nullptr, nullptr, next_w, s->y, s->y_bf, T, W, eps, st, 0.f));
+    }
+    *next_ready = fuse_next;
+    if (s->keep_on && s->keep)
+        QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)r * s->cap * W, x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    return 0;
+}
+
 // Sandwich blocks: the stream x lives in plane 1 of the stack, the embedding rows stay in plane
 // 0.  h_ready: the run's normed input is already in s->y (the previous run's last kernel made
 // it).  The last kernel of the run also makes the next run's input unless the streams are kept.
@@ -944,7 +1106,15 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     LayeredBatch* s = b->lb;
     const int W = m->a.width;
     const float* x = s->stack;
-    if (m->a.block == QIE_BLOCK_SANDWICH) {
+    const float w_one = m->a.block == QIE_BLOCK_PRENORM ? 0.f : 1.f;
+    if (m->a.block == QIE_BLOCK_PRENORM) {
+        float* xs = s->stack + s->cap * W;
+        QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, xs, nullptr, T, W, m->a.vocab, e->stream, m->a.embed_scale,
+                                m->a.pos_embed == QIE_POS_SINUSOID ? s->row_pos : nullptr, m->pos_freq));
+        bool ready = false;
+        for (int r = 0; r < (int)m->runs.size(); r++) QIE_TRY(enq_run_prenorm(b, r, T, ready, &ready));
+        x = xs;
+    } else if (m->a.block == QIE_BLOCK_SANDWICH) {
         // the embedding rows stay in plane 0 only when a repeated group adds them again
         float* xs = s->stack + s->cap * W;
         QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, m->loops ? s->stack : xs, nullptr, T, W, m->a.vocab, e->stream));
@@ -960,7 +1130,7 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
         for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, x_bf, T, &x, &x_bf));
     }
     if (n_want > 0) {
-        QIE_TRY(lay::final_rows(x, s->want, s->xn, s->xn_bf, n_want, W, m->g_final, m->w_final, m->a.norm_eps, e->stream));
+        QIE_TRY(lay::final_rows(x, s->want, s->xn, s->xn_bf, n_want, W, m->g_final, m->w_final, m->a.norm_eps, e->stream, w_one));
         QIE_TRY(dense(b, s->xn, W, m->head, s->logits, m->a.vocab, n_want, m->a.vocab, W, s->xn_bf));
     }
     return 0;
@@ -1150,6 +1320,7 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     s->v_transposed = !m->f32;
     for (int i = 0; i < m->a.n_layers; i++) {
         const qie_layer_desc& d = m->L[i].d;
+        if (d.mixer == QIE_MIXER_MINGRU) continue;   // caches nothing
         if (d.mixer == QIE_MIXER_LATENT_ATTENTION || !lay::gqa_attention_mfma_fits(d.gqa.dim, d.gqa.vdim, page_tokens))
             s->v_transposed = false;
         if (d.mixer != QIE_MIXER_LATENT_ATTENTION) s->m_vd = std::max<int64_t>(s->m_vd, d.gqa.vdim);
@@ -1158,7 +1329,17 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     for (int r = 0; r < n_runs; r++) {
         const int i = m->runs[r].layer;
         const qie_layer_desc& d = m->L[i].d;
-        if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
+        if (d.mixer == QIE_MIXER_MINGRU) {
+            // no cache rows; `width` state elements per slot
+            const int64_t n = d.mingru.width;
+            s->state_off[r] = s->slot_state;
+            s->slot_state += n;
+            s->m_state = std::max<int64_t>(s->m_state, n);
+            s->m_hd = std::max<int64_t>(s->m_hd, n);
+            s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
+            s->m_hv = std::max<int64_t>(s->m_hv, n);
+            s->m_abf = std::max<int64_t>({s->m_abf, (int64_t)m->a.width, n});
+        } else if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
             // K rows, then V rows of this run; one state per slot for the recurrence
             const qie_gqa_desc& a = d.gqa;
             s->layer_off[r] = off;
@@ -1189,7 +1370,7 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
             }
             if (d.ff_kind == QIE_FF_MOE) {
                 s->m_top = std::max<int64_t>(s->m_top, d.top);
-                s->m_e = std::max<int64_t>(s->m_e, d.experts);
+                s->m_e = std::max<int64_t>(s->m_e, d.experts + (d.router == QIE_ROUTER_SOFTMAX_ALL ? d.identity : 0));
             }
             continue;
         }
@@ -1278,8 +1459,13 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
                 "qie_engine_create_layered: invalid sizes");
     QIE_REQUIRE(!opts || !opts->tp_comm, "qie_engine_create_layered: layered engines run on one device");
     QIE_REQUIRE(!opts || (!opts->weight_fp8 && !opts->prefill_fp8), "qie_engine_create_layered: fp8 weights are not covered");
-    QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN || arch->block == QIE_BLOCK_SANDWICH, "qie_engine_create_layered: block %d",
+    QIE_REQUIRE(arch->block >= QIE_BLOCK_POSTNORM_GAIN && arch->block <= QIE_BLOCK_PRENORM, "qie_engine_create_layered: block %d",
                 arch->block);
+    QIE_REQUIRE(arch->pos_embed == QIE_POS_NONE || arch->pos_embed == QIE_POS_SINUSOID, "qie_engine_create_layered: positions %d",
+                arch->pos_embed);
+    QIE_REQUIRE((arch->pos_embed == QIE_POS_NONE && (arch->embed_scale == 0.f || arch->embed_scale == 1.f)) ||
+                    arch->block == QIE_BLOCK_PRENORM,
+                "qie_engine_create_layered: scaled embeddings and position vectors go with the pre-norm block");
     QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN || !arch->depth_mix,
                 "qie_engine_create_layered: depth-weighted residuals go with the post-norm block");
     const bool loops = arch->loop_times > 1 && arch->loop_stop > arch->loop_start;
@@ -1293,10 +1479,29 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
         QIE_REQUIRE(d.ff_kind == QIE_FF_NONE || d.ff > 0, "layer %d: feed-forward size", i);
         QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts), "layer %d: %d of %d experts", i,
                     d.top, d.experts);
-        QIE_REQUIRE(d.router == QIE_ROUTER_SIGMOID_IN || d.router == QIE_ROUTER_SOFTMAX_OUT, "layer %d: router %d", i, d.router);
+        QIE_REQUIRE(d.router >= QIE_ROUTER_SIGMOID_IN && d.router <= QIE_ROUTER_SOFTMAX_ALL, "layer %d: router %d", i, d.router);
+        QIE_REQUIRE(d.ff_act == QIE_ACT_SILU_GATED || d.ff_act == QIE_ACT_XIELU, "layer %d: activation %d", i, d.ff_act);
+        if (d.ff_kind == QIE_FF_MOE && d.router == QIE_ROUTER_SOFTMAX_ALL) {
+            const int n = d.experts + d.identity;
+            QIE_REQUIRE(d.identity >= 0 && d.groups >= 1 && n % d.groups == 0 && d.groups_keep >= 1 && d.groups_keep <= d.groups &&
+                            d.top <= d.groups_keep * (n / d.groups),
+                        "layer %d: %d + %d router outputs in %d groups, %d kept, top %d", i, d.experts, d.identity, d.groups,
+                        d.groups_keep, d.top);
+        } else {
+            QIE_REQUIRE(d.identity == 0, "layer %d: identity experts go with the grouped softmax router", i);
+        }
+        if (d.mixer == QIE_MIXER_MINGRU) {
+            QIE_REQUIRE(arch->block == QIE_BLOCK_PRENORM, "layer %d: this mixer is wired to the pre-norm block", i);
+            QIE_REQUIRE(d.mingru.width > 0, "layer %d: minGRU width", i);
+            continue;
+        }
         if (d.mixer == QIE_MIXER_GQA || d.mixer == QIE_MIXER_GQA_RECURRENT) {
             const qie_gqa_desc& a = d.gqa;
-            QIE_REQUIRE(arch->block == QIE_BLOCK_SANDWICH, "layer %d: this mixer is wired to the sandwich block", i);
+            QIE_REQUIRE(arch->block == QIE_BLOCK_SANDWICH || (arch->block == QIE_BLOCK_PRENORM && d.mixer == QIE_MIXER_GQA),
+                        "layer %d: this mixer is wired to the sandwich block (alone: also the pre-norm block)", i);
+            QIE_REQUIRE(a.weights == QIE_WEIGHTS_SOFTMAX || a.weights == QIE_WEIGHTS_SIGMOID, "layer %d: attention weights %d", i,
+                        a.weights);
+            QIE_REQUIRE(a.q_temp_every >= 0, "layer %d: query temperature every %d", i, a.q_temp_every);
             QIE_REQUIRE(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0 && a.dim > 0 && a.vdim > 0,
                         "layer %d: %d query heads over %d key heads of %d / %d", i, a.heads, a.kv_heads, a.dim, a.vdim);
             QIE_REQUIRE(a.qk_norm >= QIE_QKNORM_NONE && a.qk_norm <= QIE_QKNORM_PLAIN, "layer %d: q / k norm %d", i, a.qk_norm);
@@ -1402,7 +1607,14 @@ int qie_engine_finalize_weights(qie_engine* e) {
         QIE_TRY(lm_alloc(m, &m->head, (size_t)V * W * m->esz()));
         QIE_TRY(lm_upload_rows(m, m->head, 0, W, *th));
     }
-    if (m->a.block == QIE_BLOCK_SANDWICH) {
+    if (m->a.embed_scale == 0.f) m->a.embed_scale = 1.f;
+    if (m->a.pos_embed == QIE_POS_SINUSOID) {
+        std::vector<double> fr((size_t)(W + 1) / 2);
+        for (size_t i = 0; i < fr.size(); i++) fr[i] = std::pow(10000.0, -2.0 * (double)i / (double)W);
+        QIE_TRY(lm_alloc(m, (void**)&m->pos_freq, fr.size() * 8));
+        QIE_HIP(hipMemcpy(m->pos_freq, fr.data(), fr.size() * 8, hipMemcpyHostToDevice));
+    }
+    if (m->a.block == QIE_BLOCK_SANDWICH || m->a.block == QIE_BLOCK_PRENORM) {
         QIE_TRY(lm_vector(m, &m->w_final, "final.norm", W));
     } else {
         LM_GET(tn, "final.norm");
@@ -1604,7 +1816,9 @@ int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t ite
     QIE_HIP(hipEventCreate(&e1));
     int rc = 0;
     const bool gqa = which != 0 && m->L[layer].d.mixer != QIE_MIXER_LATENT_ATTENTION;
-    QIE_REQUIRE(which != 4 || m->L[layer].d.mixer == QIE_MIXER_GQA_RECURRENT, "qie_batch_time_stage: layer %d has no recurrence", layer);
+    QIE_REQUIRE(which != 4 || m->L[layer].d.mixer == QIE_MIXER_GQA_RECURRENT || m->L[layer].d.mixer == QIE_MIXER_MINGRU,
+                "qie_batch_time_stage: layer %d has no recurrence", layer);
+    QIE_REQUIRE(which != 1 || m->L[layer].d.mixer != QIE_MIXER_MINGRU, "qie_batch_time_stage: layer %d has no attention", layer);
     int run = 0;   // the layer's first run
     while (which != 0 && m->runs[run].layer != layer) run++;
     auto once = [&]() -> int {
@@ -1617,7 +1831,7 @@ int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t ite
                     QIE_TRY(enq_gqa_proj(b, run, T));
                     return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
                 case 3: return enq_ff(b, layer, T);
-                default: return enq_recurrence(b, run, T);
+                default: return L.d.mixer == QIE_MIXER_MINGRU ? enq_mingru(b, run, T) : enq_recurrence(b, run, T);
             }
         }
         switch (which) {

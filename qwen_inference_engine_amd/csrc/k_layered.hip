@@ -270,24 +270,33 @@ int linear(const LinearP& p, bool w_f32, hipStream_t st) {
 }
 
 // ------------------------------------------------------------------ embedding rows
+// out[t] = E[tok[t]] * scale (+ the sinusoidal vector of the row's position when pos: entry 2i =
+// sin(pos * freq[i]), entry 2i + 1 = cos of the same; freq and the angle in double, rounded once)
 template <typename TW>
 __global__ __launch_bounds__(256) void embed_rows_kernel(const TW* E, const int32_t* tok, float* out, uint16_t* out_bf, int W,
-                                                         int vocab) {
+                                                         int vocab, float scale, const int32_t* pos, const double* freq) {
     const int t = blockIdx.x;
     int id = tok[t];
     if (id < 0 || id >= vocab) id = 0;
     for (int w = threadIdx.x; w < W; w += 256) {
-        const float v = ldf<TW>(E, (int64_t)id * W + w);
+        float v = ldf<TW>(E, (int64_t)id * W + w) * scale;
+        if (pos) {
+            const double ang = (double)pos[t] * freq[w >> 1];
+            v += (float)((w & 1) ? cos(ang) : sin(ang));
+        }
         out[(int64_t)t * W + w] = v;
         if (out_bf) out_bf[(int64_t)t * W + w] = f2bf(v);
     }
 }
 int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16_t* out_bf, int T, int W, int vocab,
-               hipStream_t st) {
+               hipStream_t st, float scale, const int32_t* pos, const double* freq) {
+    QIE_REQUIRE(!pos || freq, "embed_rows: positions without their frequencies");
     if (w_f32)
-        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)E, tok, out, out_bf, W, vocab);
+        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)E, tok, out, out_bf, W, vocab, scale, pos,
+                           freq);
     else
-        hipLaunchKernelGGL(embed_rows_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)E, tok, out, out_bf, W, vocab);
+        hipLaunchKernelGGL(embed_rows_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)E, tok, out, out_bf, W, vocab,
+                           scale, pos, freq);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -491,7 +500,7 @@ int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T
 
 // rows picked by index, normed with one gain: out[i] = gain * x[rows[i]] / rms
 __global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int W,
-                                                         float gain, const float* w1p, float eps) {
+                                                         float gain, const float* w1p, float eps, float w_one) {
     __shared__ float red[4];
     const int64_t t = rows[blockIdx.x];
     float ss = 0.f;
@@ -502,14 +511,14 @@ __global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const i
     ss = block_sum256(ss, red);
     const float inv = gain / sqrtf(ss / (float)W + eps);
     for (int i = threadIdx.x; i < W; i += 256) {
-        const float o = x[t * W + i] * inv * (w1p ? 1.0f + w1p[i] : 1.0f);
+        const float o = x[t * W + i] * inv * (w1p ? w_one + w1p[i] : 1.0f);
         out[(int64_t)blockIdx.x * W + i] = o;
         if (out_bf) out_bf[(int64_t)blockIdx.x * W + i] = f2bf(o);
     }
 }
 int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, const float* w1p,
-               float eps, hipStream_t st) {
-    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, out_bf, W, gain, w1p, eps);
+               float eps, hipStream_t st, float w_one) {
+    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, out_bf, W, gain, w1p, eps, w_one);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -548,6 +557,23 @@ int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipSt
     const int64_t n = M * ff;
     if (n == 0) return 0;
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, a_bf, ff, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// a = xielu(u): ap u^2 + u / 2 for u > 0, else aq (exp(u) - 1 - u) + u / 2 (ap = softplus(p),
+// aq = 1/2 + softplus(q), made once on the host)
+__global__ __launch_bounds__(256) void xielu_kernel(const float* u, float* a, uint16_t* a_bf, float ap, float aq, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float z = u[i];
+    const float o = z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(aq, expm1f(z) - z, 0.5f * z);
+    a[i] = o;
+    if (a_bf) a_bf[i] = f2bf(o);
+}
+int xielu(const float* u, float* a, uint16_t* a_bf, int64_t n, float ap, float aq, hipStream_t st) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(xielu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, u, a, a_bf, ap, aq, n);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -604,6 +630,85 @@ int route_topk(const float* y, const void* Wr, const float* bias, bool w_f32, in
     else
         hipLaunchKernelGGL(route_kernel<uint16_t>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const uint16_t*)Wr, bias, W, E, top,
                            mode, sel, score);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// Router over all E outputs (real and identity experts alike): s = softmax(z) in fp32; the choice
+// ranks s + corr; a group of E / groups neighbours ranks by its largest choice score and only the
+// `keep` best groups stay eligible (the others count as minus infinity); the `top` best eligible
+// are chosen, weighted by s / (sum of the chosen s + 1e-20) * scale.  Ties: the lower index.
+// One block per row; shared: s [E], choice [E], group rank [groups].
+template <typename TW>
+__global__ __launch_bounds__(256) void route_grouped_kernel(const float* y, const TW* Wr, const float* corr, int W, int E, int top,
+                                                            int groups, int keep, float scale, int32_t* sel, float* score) {
+    extern __shared__ float sh[];
+    float* s = sh;
+    float* ch = sh + E;
+    float* gs = ch + E;
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int e = wave; e < E; e += 4) {
+        float z = 0.f;
+        for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
+        z = wave_sum(z);
+        if (lane == 0) s[e] = z;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    float mx = s[0];
+    for (int e = 1; e < E; e++) mx = fmaxf(mx, s[e]);
+    float den = 0.f;
+    for (int e = 0; e < E; e++) {
+        s[e] = expf(s[e] - mx);
+        den += s[e];
+    }
+    for (int e = 0; e < E; e++) {
+        s[e] = s[e] / den;
+        ch[e] = s[e] + corr[e];
+    }
+    const int per = E / groups;
+    for (int g = 0; g < groups; g++) {
+        float b = ch[g * per];
+        for (int e = 1; e < per; e++) b = fmaxf(b, ch[g * per + e]);
+        gs[g] = b;
+    }
+    for (int g = 0; g < groups; g++) {   // a group stays when fewer than `keep` groups rank before it
+        int before = 0;
+        for (int o = 0; o < groups; o++) before += (gs[o] > gs[g]) || (gs[o] == gs[g] && o < g);
+        if (before >= keep)
+            for (int e = 0; e < per; e++) ch[g * per + e] = -INFINITY;
+    }
+    float sum = 0.f;
+    for (int k = 0; k < top; k++) {
+        int best = -1;
+        float bv = 0.f;
+        for (int e = 0; e < E; e++)
+            if (ch[e] != -INFINITY && (best < 0 || ch[e] > bv)) {
+                bv = ch[e];
+                best = e;
+            }
+        if (best < 0) best = 0;   // only if scores are not finite
+        sel[t * top + k] = best;
+        score[t * top + k] = s[best];
+        sum += s[best];
+        ch[best] = -INFINITY;
+    }
+    const float inv = scale / (sum + 1e-20f);
+    for (int k = 0; k < top; k++) score[t * top + k] *= inv;
+}
+int route_grouped(const float* y, const void* Wr, const float* corr, bool w_f32, int T, int W, int E, int top, int groups, int keep,
+                  float scale, int32_t* sel, float* score, hipStream_t st) {
+    QIE_REQUIRE(top >= 1 && top <= E && E <= 4096 && corr, "router: top %d of %d outputs", top, E);
+    QIE_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (E / groups),
+                "router: %d groups of %d outputs, %d kept, top %d", groups, E, keep, top);
+    const size_t shm = (size_t)(2 * E + groups) * 4;
+    if (w_f32)
+        hipLaunchKernelGGL(route_grouped_kernel<float>, dim3(T), dim3(256), shm, st, y, (const float*)Wr, corr, W, E, top, groups, keep,
+                           scale, sel, score);
+    else
+        hipLaunchKernelGGL(route_grouped_kernel<uint16_t>, dim3(T), dim3(256), shm, st, y, (const uint16_t*)Wr, corr, W, E, top,
+                           groups, keep, scale, sel, score);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -673,21 +778,29 @@ int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T
     QIE_LAUNCH_CHECK();
     return 0;
 }
-// f[t, :] = sum_k (score[t * top + k] or 1) * yd[slot_of[t * top + k], :]
+// f[t, :] = sum_k (score[t * top + k] or 1) * yd[slot_of[t * top + k], :]; a chosen expert >= n_real (when
+// sel) is an identity expert: its output is the row's input y[t, :]
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* yd, const int32_t* slot_of, const float* score, int top, int W,
-                                                          float* f) {
+                                                          float* f, const int32_t* sel, int n_real, const float* y) {
     const int64_t t = blockIdx.x;
     for (int w = threadIdx.x; w < W; w += 256) {
         float s = 0.f;
-        if (score)
+        if (sel)
+            for (int k = 0; k < top; k++) {
+                const float o = sel[t * top + k] >= n_real ? y[t * W + w] : yd[(int64_t)slot_of[t * top + k] * W + w];
+                s = fmaf(score ? score[t * top + k] : 1.0f, o, s);
+            }
+        else if (score)
             for (int k = 0; k < top; k++) s = fmaf(score[t * top + k], yd[(int64_t)slot_of[t * top + k] * W + w], s);
         else
             for (int k = 0; k < top; k++) s += yd[(int64_t)slot_of[t * top + k] * W + w];
         f[t * W + w] = s;
     }
 }
-int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st) {
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, yd, slot_of, score, top, W, f);
+int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st,
+                const int32_t* sel, int n_real, const float* y) {
+    QIE_REQUIRE(!sel || y, "moe_combine: identity experts need the rows' input");
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, yd, slot_of, score, top, W, f, sel, n_real, y);
     QIE_LAUNCH_CHECK();
     return 0;
 }

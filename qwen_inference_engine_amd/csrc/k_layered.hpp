@@ -126,6 +126,10 @@ struct GqaPostP {
     LatentCache cache;
     int64_t k_off, v_off;
     int v_transposed;         // V rows of a page stored [kv_heads][vdim][page_tokens]
+    // q_temp_every > 0: the normed query is multiplied by 1 + q_temp_coef * ln((pos + 1) / every + 1),
+    // the division rounded down
+    int q_temp_every;
+    float q_temp_coef;
 };
 int gqa_post(const GqaPostP& p, bool cache_f32, int T, hipStream_t st);
 
@@ -156,6 +160,10 @@ struct GqaAttnP {
     uint16_t* out_bf;
     int64_t ld_out;
     int out_col;
+    const float* slopes;      // [heads] or null: the score also loses slopes[h] * (i - j)
+    const float* pb;          // [heads] or null; set: a visible key's weight is sigmoid(score + pb[h]),
+                              // not normalised over the keys (no softmax)
+    int gate_col;             // >= 0: head h's result times sigmoid(proj[t * ld + gate_col + h])
 };
 int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);
 // The matrix-core form for bf16 caches whose V rows are stored transposed (v_transposed: inside a
@@ -226,34 +234,88 @@ struct GatedCarryP {
 };
 int gated_carry(const GatedCarryP& p, hipStream_t st);
 // out[t, out_col + h * vdim + c] = scale * o[t, h, c] / sqrt(mean_c o^2 + eps) * w[c], o = o1 + o2 when o2
+// ------------------------------------------------------------------ minGRU
+// Per entry {first packed row, rows, index, first position} and channel c < n: with
+// z = sigmoid(proj[z_col + c] + z_b[c]), u = proj[x_col + c] + x_b[c], cand = u >= 0 ? u + 1/2 :
+// sigmoid(u), the state runs through the entry's rows in order, S = (1 - z) S + z cand, and
+// out[row, c] = S * silu(proj[g_col + c]) (with its bf16 image).  fp32 throughout.
+// init: the state an entry starts from, at init + index * init_stride (+ init_off); null, or (when
+// init_if_pos) an entry whose first position is 0: zero.  end / decay (optional, same addressing
+// with end_stride): the state after the entry's last row, the product of its (1 - z).  out may be
+// null (a pass that only wants end and decay).
+struct MinGruScanP {
+    const float* proj;
+    int64_t ld;
+    int z_col, x_col, g_col;
+    const float* z_b;
+    const float* x_b;
+    const int4* entries;
+    int n_entries, n;
+    const float* init;
+    int64_t init_stride, init_off;
+    int init_if_pos;
+    float* end;
+    float* decay;
+    int64_t end_stride, end_off;
+    float* out;
+    uint16_t* out_bf;
+    int64_t ld_out;
+};
+int mingru_scan(const MinGruScanP& p, hipStream_t st);
+// Long entries in pieces (lists as for gated_carry): s_in[c] = the state entering piece c, from the
+// slot's state (or zero at position 0) through S <- decay[c] S + s_loc[c]; the slot's state = what
+// leaves the entry's last piece.
+struct MinGruCarryP {
+    const int4* spans;
+    int n_spans, n;
+    const float* s_loc;
+    const float* decay;
+    float* s_in;
+    float* state;
+    int64_t slot_stride, state_off;
+};
+int mingru_carry(const MinGruCarryP& p, hipStream_t st);
+
 int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
                    uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st);
-// Rows of W: x = xin + rms(v) * (1 + wb) (when v) + add (when add); then (when wn)
-// h = rms(x) * (1 + wn) with its bf16 image.  xin may be x.
+// Rows of W: x = xin + (wb ? rms(v) * (w_one + wb) : v) (when v) + add (when add); then (when wn)
+// h = rms(x) * (w_one + wn) with its bf16 image.  xin may be x.  w_one = 1: weight vectors stored
+// around zero; 0: plain weights.
 int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,
-             int T, int W, float eps, hipStream_t st);
+             int T, int W, float eps, hipStream_t st, float w_one = 1.0f);
 
 // The producers below also write the bf16 image of their result when the *_bf pointer is set
 // (bf16 engines: the next product reads it; no separate rounding pass).
+// out[t] = E[tok[t]] * scale; with pos (the rows' positions) and freq (double [ceil(W / 2)]) the
+// sinusoidal position vector is added: entry 2i = sin(pos * freq[i]), entry 2i + 1 = cos of it
 int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16_t* out_bf, int T, int W, int vocab,
-               hipStream_t st);
+               hipStream_t st, float scale = 1.0f, const int32_t* pos = nullptr, const double* freq = nullptr);
 int head_gate(float* v, uint16_t* v_bf, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);
 // y = (x ? x : 0) + gain * v / sqrt(mean(v^2) + eps), rows of W
 int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T, int W, float gain, float eps, hipStream_t st);
-// out[i] = gain * rms(x[rows[i]]) (* (1 + w1p) when w1p)
+// out[i] = gain * rms(x[rows[i]]) (* (w_one + w1p) when w1p)
 int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, const float* w1p,
-               float eps, hipStream_t st);
+               float eps, hipStream_t st, float w_one = 1.0f);
 int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, uint16_t* x_bf, int64_t count, hipStream_t st);
 int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st);
+// a = ap u^2 + u / 2 where u > 0, else aq (exp(u) - 1 - u) + u / 2; n elements
+int xielu(const float* u, float* a, uint16_t* a_bf, int64_t n, float ap, float aq, hipStream_t st);
 // mode 0: score = sigmoid(z) of the `top` largest z = W_r y; mode 1: z = W_r y + bias, score = the
 // softmax over the `top` largest z alone.  Ties: the lower index.
 int route_topk(const float* y, const void* Wr, const float* bias, bool w_f32, int T, int W, int E, int top, int mode, int32_t* sel,
                float* score, hipStream_t st);
+// s = softmax over all E router outputs; chosen by s + corr inside the `keep` best of `groups` equal
+// groups of neighbours (a group ranks by its largest s + corr), `top` of them; score = s of the
+// chosen / (their sum + 1e-20) * scale.  Ties: the lower index.
+int route_grouped(const float* y, const void* Wr, const float* corr, bool w_f32, int T, int W, int E, int top, int groups, int keep,
+                  float scale, int32_t* sel, float* score, hipStream_t st);
 int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st);
 // score (may be null: 1) scales the gathered input rows / the combined output rows
 int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, uint16_t* xg_bf,
                hipStream_t st);
-int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st);
+// sel / n_real / y: a chosen expert >= n_real is an identity expert whose output is the row's input y
+int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st,
+                const int32_t* sel = nullptr, int n_real = 0, const float* y = nullptr);
 int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st);
 int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
 int rows_to_bf16_strided(const float* x, int64_t ldx, uint16_t* y, int64_t ldy, int64_t M, int K, hipStream_t st);

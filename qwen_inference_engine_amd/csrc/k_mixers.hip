@@ -5,7 +5,10 @@
 //   lay::gqa_attention   grouped-query softmax attention over the paged rows with a causal,
 //                        sliding or block-local mask and an optional log-distance bias; the
 //                        weighted sum of turned values is turned back
+//                        and / or a linear one with a slope per head; softmax weights, or sigmoid
+//                        weights with a bias per head; an optional sigmoid gate per head
 //   lay::gated_scan      gated linear recurrence with an fp32 state per slot and head
+//   lay::mingru_scan     minGRU: a gated recurrence per channel whose gates read the current token
 //   lay::head_norm_rows  per-head RMS norm with a weight
 //   lay::add_norm        residual add of a normed branch fused with the next branch's input norm
 //
@@ -119,6 +122,10 @@ __global__ __launch_bounds__(256) void gqa_post_kernel(GqaPostP p) {
                 const float* w = p.qk_norm == 1 ? (is_q ? p.qn_w : p.kn_w) : nullptr;
                 for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * (w ? w[i] : 1.0f);
             }
+            if (is_q && p.q_temp_every > 0) {
+                const float tq = 1.0f + p.q_temp_coef * logf((float)((pos + 1) / p.q_temp_every + 1));
+                for (int i = lane; i < dim; i += 64) buf[i] *= tq;
+            }
         }
         __syncthreads();
         if (on)
@@ -190,6 +197,9 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
     __syncthreads();
     const int lo = first_visible(p.mask, p.mask_size, pos);
     const float b1 = p.r1 ? p.r1[h] : 0.f, b2 = p.r1 ? p.r2[h] : 0.f;
+    const float slope = p.slopes ? p.slopes[h] : 0.f;
+    const bool sig = p.pb != nullptr;
+    const float pbh = sig ? p.pb[h] : 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     float acc[GA_MAXV] = {};
     for (int j0 = lo; j0 <= pos; j0 += GA_CHUNK) {
@@ -204,10 +214,28 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
             if (lane == 0) {
                 s *= p.scale;
                 if (p.r1) s -= b1 * log1pf(b2 * (float)(pos - j));
-                sc[jj] = s;
+                if (p.slopes) s -= slope * (float)(pos - j);
+                sc[jj] = sig ? 1.0f / (1.0f + expf(-(s + pbh))) : s;
             }
         }
         __syncthreads();
+        if (sig) {   // the weights are final: no running maximum, no normalisation
+            for (int jj = 0; jj < nk; jj++) {
+                const int j = j0 + jj;
+                const int pt = j % p.cache.page_tokens;
+                const TC* v = (const TC*)p.cache.pool + page_base(p.cache, slot, j) + p.v_off;
+                const float w = sc[jj];
+#pragma unroll
+                for (int i = 0; i < GA_MAXV; i++) {
+                    const int r = tid + i * 256;
+                    if (r < vdim)
+                        acc[i] = fmaf(w, ldc<TC>(v, p.v_transposed ? ((int64_t)g * vdim + r) * p.cache.page_tokens + pt
+                                                                     : ((int64_t)pt * G + g) * vdim + r), acc[i]);
+                }
+            }
+            __syncthreads();
+            continue;
+        }
         float mx = -INFINITY;
         for (int jj = tid; jj < nk; jj += 256) mx = fmaxf(mx, sc[jj]);
         mx = wmax(mx);
@@ -243,7 +271,8 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
         }
         __syncthreads();
     }
-    const float inv = 1.0f / l_run;
+    float inv = sig ? 1.0f : 1.0f / l_run;
+    if (p.gate_col >= 0) inv *= 1.0f / (1.0f + expf(-p.proj[(int64_t)t * p.ld + p.gate_col + h]));
 #pragma unroll
     for (int i = 0; i < GA_MAXV; i++) {
         const int r = tid + i * 256;
@@ -343,6 +372,14 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
     }
 }
 
+// What a column's value sums are multiplied by: 1 / (sum of its softmax weights), or 1 for sigmoid
+// weights; times the head's sigmoid gate when the mixer has one.
+__device__ __forceinline__ float gqa_out_factor(const GqaAttnP& a, float l, int row, int hh) {
+    float f = a.pb ? 1.0f : 1.0f / l;
+    if (a.gate_col >= 0) f *= 1.0f / (1.0f + __expf(-a.proj[(int64_t)row * a.ld + a.gate_col + hh]));
+    return f;
+}
+
 // SHARE: the four waves of a workgroup are four heads of one key head (heads / kv_heads a
 // multiple of 4, one head per wave whatever the group's size): every 32-key K tile and V^T tile
 // is brought to LDS once per workgroup (next tile in registers meanwhile) and each wave takes
@@ -386,10 +423,13 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
     const int S = P.S, z = blockIdx.z;
     const int bs = b0 + (int)((int64_t)nb * z / S), be = b0 + (int)((int64_t)nb * (z + 1) / S);
     const float b1 = a.r1 ? a.r1[hh] : 0.f, b2 = a.r1 ? a.r2[hh] : 0.f;
+    const float slope = a.slopes ? a.slopes[hh] : 0.f;
+    const bool sig = a.pb != nullptr;   // sigmoid weights: final as computed, no running maximum or sum
+    const float pbh = sig ? a.pb[hh] : 0.f;
     const int PT = a.cache.page_tokens;
     const uint16_t* pool = (const uint16_t*)a.cache.pool;
     const int32_t* tab = a.cache.table + (int64_t)slot * a.cache.max_pages;
-    float m_run = -1e30f, l_run = 0.f;
+    float m_run = sig ? 0.f : -1e30f, l_run = sig ? 1.f : 0.f;
     gf32x4_t acc[DV];
 #pragma unroll
     for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -486,28 +526,37 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
             vis[e] = valid && kj >= lo_q && kj <= qpos;
             float x = sacc[e >> 2][e & 3] * a.scale;
             if (a.r1) x -= b1 * __logf(1.0f + b2 * (float)max(qpos - kj, 0));
+            x -= slope * (float)max(qpos - kj, 0);
             s[e] = vis[e] ? x : -1e30f;
             bm = fmaxf(bm, s[e]);
         }
-        bm = xg_max(bm);
-        const float m_new = fmaxf(m_run, bm);
-        const float alpha = __expf(m_run - m_new);
-        float ls = 0.f, pv[8];
+        float alpha = 1.0f, pv[8];
+        if (sig) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            pv[e] = vis[e] ? __expf(s[e] - m_new) : 0.f;
-            ls += pv[e];
+            for (int e = 0; e < 8; e++) pv[e] = vis[e] ? 1.0f / (1.0f + __expf(-(s[e] + pbh))) : 0.f;
+        } else {
+            bm = xg_max(bm);
+            const float m_new = fmaxf(m_run, bm);
+            alpha = __expf(m_run - m_new);
+            float ls = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                pv[e] = vis[e] ? __expf(s[e] - m_new) : 0.f;
+                ls += pv[e];
+            }
+            ls = xg_sum(ls);
+            l_run = l_run * alpha + ls;
+            m_run = m_new;
         }
-        ls = xg_sum(ls);
-        l_run = l_run * alpha + ls;
-        m_run = m_new;
         const uint4 pu = make_uint4(pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7]));
         const gbf16x8_t pf = __builtin_bit_cast(gbf16x8_t, pu);
 #pragma unroll
         for (int dv = 0; dv < DV; dv++) {
             const uint4 vu = make_uint4(vf[dv][0].x, vf[dv][0].y, vf[dv][1].x, vf[dv][1].y);
+            if (!sig) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[dv][j] *= alpha;
+                for (int j = 0; j < 4; j++) acc[dv][j] *= alpha;
+            }
             acc[dv] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, vu), pf, acc[dv], 0, 0, 0);
         }
         if (!SHARE) {
@@ -519,7 +568,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
     }
     if (!active) return;
     if (S == 1) {
-        if (valid) gqa_store<DV>(a, acc, 1.0f / l_run, row, hh, qpos, g);
+        if (valid) gqa_store<DV>(a, acc, gqa_out_factor(a, l_run, row, hh), row, hh, qpos, g);
         return;
     }
     const int64_t unit = ((int64_t)blockIdx.x * (gridDim.y * 4) + tile) * S + z;
@@ -576,7 +625,7 @@ __global__ __launch_bounds__(256) void gqa_attn_combine_kernel(GqaAttnMfmaP P, i
             acc[dv][3] += o0[dv].w * w0 + o1[dv].w * w1;
         }
     }
-    gqa_store<DV>(a, acc, 1.0f / L, grp.x + tI, hh, pos0 + tI, g);
+    gqa_store<DV>(a, acc, gqa_out_factor(a, L, grp.x + tI, hh), grp.x + tI, hh, pos0 + tI, g);
 }
 
 bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens) {
@@ -801,6 +850,74 @@ int gated_carry(const GatedCarryP& p, hipStream_t st) {
     return 0;
 }
 
+// ------------------------------------------------------------------ minGRU
+// One thread per (entry, channel); the entry's rows go through in order, the loads of a few rows
+// ahead are independent of the recurrence, so they overlap it.
+__global__ __launch_bounds__(256) void mingru_scan_kernel(MinGruScanP p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.n) return;
+    const int4 en = p.entries[blockIdx.y];
+    float S = 0.f;
+    if (p.init && (!p.init_if_pos || en.w > 0)) S = p.init[(int64_t)en.z * p.init_stride + p.init_off + c];
+    const float zb = p.z_b[c], xb = p.x_b[c];
+    float run = 1.0f;
+    const float* row = p.proj + (int64_t)en.x * p.ld;
+    constexpr int U = 4;
+    for (int t0 = 0; t0 < en.y; t0 += U) {
+        float rz[U], rx[U], rg[U];
+#pragma unroll
+        for (int k = 0; k < U; k++) {
+            const bool on = t0 + k < en.y;
+            const float* r = row + (int64_t)(on ? t0 + k : t0) * p.ld;
+            rz[k] = r[p.z_col + c];
+            rx[k] = r[p.x_col + c];
+            rg[k] = p.out ? r[p.g_col + c] : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < U; k++) {
+            if (t0 + k >= en.y) break;
+            const float z = 1.0f / (1.0f + expf(-(rz[k] + zb)));
+            const float u = rx[k] + xb;
+            const float cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
+            S = (1.0f - z) * S + z * cand;
+            run *= 1.0f - z;
+            if (p.out) {
+                const float o = S * (rg[k] / (1.0f + expf(-rg[k])));
+                const int64_t oi = (int64_t)(en.x + t0 + k) * p.ld_out + c;
+                p.out[oi] = o;
+                if (p.out_bf) p.out_bf[oi] = f2bf(o);
+            }
+        }
+    }
+    if (p.end) p.end[(int64_t)en.z * p.end_stride + p.end_off + c] = S;
+    if (p.decay) p.decay[(int64_t)en.z * p.end_stride + p.end_off + c] = run;
+}
+int mingru_scan(const MinGruScanP& p, hipStream_t st) {
+    QIE_REQUIRE(p.n_entries > 0 && p.n > 0 && p.proj && p.entries && p.z_b && p.x_b && (p.out || p.end), "mingru scan: bad arguments");
+    hipLaunchKernelGGL(mingru_scan_kernel, dim3((unsigned)((p.n + 255) / 256), (unsigned)p.n_entries), dim3(256), 0, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void mingru_carry_kernel(MinGruCarryP p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.n) return;
+    const int4 sp = p.spans[blockIdx.y];
+    float* stp = p.state + (int64_t)sp.z * p.slot_stride + p.state_off + c;
+    float S = sp.w > 0 ? *stp : 0.f;
+    for (int k = sp.x; k < sp.x + sp.y; k++) {
+        p.s_in[(int64_t)k * p.n + c] = S;
+        S = fmaf(p.decay[(int64_t)k * p.n + c], S, p.s_loc[(int64_t)k * p.n + c]);
+    }
+    *stp = S;
+}
+int mingru_carry(const MinGruCarryP& p, hipStream_t st) {
+    QIE_REQUIRE(p.n_spans > 0 && p.n > 0 && p.s_loc && p.decay && p.s_in && p.state, "mingru carry: bad arguments");
+    hipLaunchKernelGGL(mingru_carry_kernel, dim3((unsigned)((p.n + 255) / 256), (unsigned)p.n_spans), dim3(256), 0, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
 // ------------------------------------------------------------------ per-head norm
 __global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, const float* o2, const float* w, float eps, float scale,
                                                              int heads, int vdim, float* out, uint16_t* out_bf, int64_t ld_out,
@@ -835,11 +952,11 @@ int head_norm_rows(const float* o, const float* o2, const float* w, float eps, f
 
 // ------------------------------------------------------------------ residual add + next norm
 __global__ __launch_bounds__(256) void add_norm_kernel(float* x, const float* xin, const float* v, const float* wb, const float* add,
-                                                       const float* wn, float* h, uint16_t* h_bf, int W, float eps) {
+                                                       const float* wn, float* h, uint16_t* h_bf, int W, float eps, float w_one) {
     __shared__ float red[4];
     const int64_t r0 = (int64_t)blockIdx.x * W;
     float inv_v = 0.f;
-    if (v) {
+    if (v && wb) {
         float ss = 0.f;
         for (int i = threadIdx.x; i < W; i += 256) {
             const float a = v[r0 + i];
@@ -851,7 +968,7 @@ __global__ __launch_bounds__(256) void add_norm_kernel(float* x, const float* xi
     float sx = 0.f;
     for (int i = threadIdx.x; i < W; i += 256) {
         float a = xin[r0 + i];
-        if (v) a += v[r0 + i] * inv_v * (1.0f + wb[i]);
+        if (v) a += wb ? v[r0 + i] * inv_v * (w_one + wb[i]) : v[r0 + i];
         if (add) a += add[r0 + i];
         if (v || add || xin != x) x[r0 + i] = a;
         sx += a * a;
@@ -860,15 +977,15 @@ __global__ __launch_bounds__(256) void add_norm_kernel(float* x, const float* xi
     sx = bsum256(sx, red);
     const float inv_x = 1.0f / sqrtf(sx / (float)W + eps);
     for (int i = threadIdx.x; i < W; i += 256) {
-        const float o = x[r0 + i] * inv_x * (1.0f + wn[i]);   // the thread's own store above
+        const float o = x[r0 + i] * inv_x * (w_one + wn[i]);   // the thread's own store above
         h[r0 + i] = o;
         if (h_bf) h_bf[r0 + i] = f2bf(o);
     }
 }
 int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,
-             int T, int W, float eps, hipStream_t st) {
-    QIE_REQUIRE(x && xin && (!v || wb) && (!wn || h), "add_norm: bad arguments");
-    hipLaunchKernelGGL(add_norm_kernel, dim3(T), dim3(256), 0, st, x, xin, v, wb, add, wn, h, h_bf, W, eps);
+             int T, int W, float eps, hipStream_t st, float w_one) {
+    QIE_REQUIRE(x && xin && (!wn || h), "add_norm: bad arguments");
+    hipLaunchKernelGGL(add_norm_kernel, dim3(T), dim3(256), 0, st, x, xin, v, wb, add, wn, h, h_bf, W, eps, w_one);
     QIE_LAUNCH_CHECK();
     return 0;
 }

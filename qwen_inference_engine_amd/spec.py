@@ -203,6 +203,11 @@ class GqaAttention:
     mask_size: int = 0
     values_are_keys: bool = False
     dist_bias: bool = False
+    weights: str = "softmax"     # "softmax" | "sigmoid": sigmoid(score + a number per head), not normalised
+    slope_bias: bool = False     # the score loses 2^(-8 (h + 1) / heads) * (i - j)
+    head_gate: bool = False      # head h's output times sigmoid(W_g x)_h
+    q_temp_coef: float = 0.0     # q times 1 + coef * ln(floor((pos + 1) / every) + 1) after its norm
+    q_temp_every: int = 0        # 0: no query temperature
 
 
 @dataclasses.dataclass(frozen=True)
@@ -224,18 +229,32 @@ class AttentionWithRecurrence:
 
 
 @dataclasses.dataclass(frozen=True)
+class MinGru:
+    """Mixer: minGRU, a gated recurrence whose gates read only the current token; `width` fp32 state
+    elements per slot."""
+    width: int
+
+
+@dataclasses.dataclass(frozen=True)
 class FeedForward:
     kind: str         # "dense" or "moe"
     ff: int           # hidden size (of one expert for "moe")
     experts: int = 0
     top: int = 0
     router: str = "sigmoid_in"   # "sigmoid_in": sigmoid scores scale the input; "softmax_out":
-                                 # biased logits, softmax over the chosen ones weights the output
+                                 # biased logits, softmax over the chosen ones weights the output;
+                                 # "softmax_all": softmax over all router outputs, chosen by score +
+                                 # correction inside the best groups, renormalised, times route_scale
+    act: str = "silu_gated"      # dense: "silu_gated" (gate, up, down) | "xielu" (up, down, two numbers)
+    identity: int = 0            # "softmax_all": identity experts after the `experts` real ones
+    groups: int = 1
+    groups_keep: int = 1
+    route_scale: float = 1.0
 
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    mixer: object     # LatentAttention | GqaAttention | AttentionWithRecurrence
+    mixer: object     # LatentAttention | GqaAttention | AttentionWithRecurrence | MinGru
     mlp: Optional[FeedForward]
 
 
@@ -248,7 +267,10 @@ class LayeredSpec:
     layers: Tuple[LayerSpec, ...]
     depth_mix: bool = True
     block: str = "postnorm_gain"     # "postnorm_gain" | "sandwich" (weight-vector norms around every branch)
+                                     # | "prenorm" (one plain-weight norm before every branch)
     tied_head: bool = False
+    embed_scale: float = 1.0
+    pos_embed: str = "none"          # "none" | "sinusoid" (added to the scaled embedding row)
     loop: Optional[Tuple[int, int, int]] = None   # (start, stop, times): layers [start, stop) run `times` times
 
     @property
@@ -282,6 +304,9 @@ class LayeredSpec:
             g.rot_values = int(m.rot_values)
             g.mask = {"causal": _lib.QIE_MASK_CAUSAL, "window": _lib.QIE_MASK_WINDOW, "chunk": _lib.QIE_MASK_CHUNK}[m.mask]
             g.mask_size, g.values_are_keys, g.dist_bias = m.mask_size, int(m.values_are_keys), int(m.dist_bias)
+            g.weights = _lib.QIE_WEIGHTS_SIGMOID if m.weights == "sigmoid" else _lib.QIE_WEIGHTS_SOFTMAX
+            g.slope_bias, g.head_gate = int(m.slope_bias), int(m.head_gate)
+            g.q_temp_coef, g.q_temp_every = m.q_temp_coef, m.q_temp_every
 
         for d, L in zip(arr, self.layers):
             m = L.mixer
@@ -293,6 +318,9 @@ class LayeredSpec:
                 gqa(d.gqa, m.attn)
                 d.rec.heads, d.rec.dim, d.rec.vdim = m.rec.heads, m.rec.dim, m.rec.vdim
                 d.gqa_scale, d.rec_scale = m.attn_scale, m.rec_scale
+            elif isinstance(m, MinGru):
+                d.mixer = _lib.QIE_MIXER_MINGRU
+                d.mingru.width = m.width
             else:
                 d.mixer = _lib.QIE_MIXER_LATENT_ATTENTION
                 d.heads, d.dim, d.rot_dim, d.vdim, d.kv_rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
@@ -302,14 +330,20 @@ class LayeredSpec:
                 d.ff_kind = _lib.QIE_FF_NONE
             elif L.mlp.kind == "dense":
                 d.ff_kind, d.ff = _lib.QIE_FF_DENSE, L.mlp.ff
+                d.ff_act = _lib.QIE_ACT_XIELU if L.mlp.act == "xielu" else _lib.QIE_ACT_SILU_GATED
             else:
                 d.ff_kind, d.ff, d.experts, d.top = _lib.QIE_FF_MOE, L.mlp.ff, L.mlp.experts, L.mlp.top
-                d.router = _lib.QIE_ROUTER_SOFTMAX_OUT if L.mlp.router == "softmax_out" else _lib.QIE_ROUTER_SIGMOID_IN
+                d.router = {"sigmoid_in": _lib.QIE_ROUTER_SIGMOID_IN, "softmax_out": _lib.QIE_ROUTER_SOFTMAX_OUT,
+                            "softmax_all": _lib.QIE_ROUTER_SOFTMAX_ALL}[L.mlp.router]
+                d.identity, d.groups, d.groups_keep, d.route_scale = L.mlp.identity, L.mlp.groups, L.mlp.groups_keep, L.mlp.route_scale
         a = _lib.ArchDescC()
         a.n_layers, a.width, a.vocab, a.norm_eps = len(self.layers), self.width, self.vocab, self.norm_eps
         a.depth_mix = int(self.depth_mix)
-        a.block = _lib.QIE_BLOCK_SANDWICH if self.block == "sandwich" else _lib.QIE_BLOCK_POSTNORM_GAIN
+        a.block = {"postnorm_gain": _lib.QIE_BLOCK_POSTNORM_GAIN, "sandwich": _lib.QIE_BLOCK_SANDWICH,
+                   "prenorm": _lib.QIE_BLOCK_PRENORM}[self.block]
         a.tied_head = int(self.tied_head)
+        a.embed_scale = self.embed_scale
+        a.pos_embed = _lib.QIE_POS_SINUSOID if self.pos_embed == "sinusoid" else _lib.QIE_POS_NONE
         if self.loop:
             a.loop_start, a.loop_stop, a.loop_times = self.loop
         a.layers = arr
@@ -319,7 +353,7 @@ class LayeredSpec:
         """Checkpoint tensor names and shapes of this architecture."""
         W, out = self.width, {"embed": [self.vocab, self.width]}
         sandwich = self.block == "sandwich"
-        nshape = [W] if sandwich else []
+        nshape = [W] if self.block in ("sandwich", "prenorm") else []
 
         def gqa(q, m):
             out[q + "q"], out[q + "k"] = [m.heads * m.dim, W], [m.kv_heads * m.dim, W]
@@ -329,6 +363,10 @@ class LayeredSpec:
                 out[q + "q.norm"], out[q + "k.norm"] = [m.dim], [m.dim]
             if m.dist_bias:
                 out[q + "r1"], out[q + "r2"] = [m.heads], [m.heads]
+            if m.weights == "sigmoid":
+                out[q + "pb"] = [m.heads]
+            if m.head_gate:
+                out[q + "g"] = [m.heads, W]
             out[q + "o"] = [W, m.heads * m.vdim]
 
         for i, L in enumerate(self.layers):
@@ -348,6 +386,10 @@ class LayeredSpec:
                 out[r + "q"], out[r + "f"], out[r + "v"] = [c.heads * c.dim, W], [c.heads * c.dim, W], [c.heads * c.vdim, W]
                 out[r + "f.b"], out[r + "lower"], out[r + "norm"] = [c.heads * c.dim], [c.heads * c.dim], [c.vdim]
                 out[r + "o"] = [W, c.heads * c.vdim]
+            elif isinstance(m, MinGru):
+                q = p + "mix."
+                out.update({q + "z": [m.width, W], q + "z.b": [m.width], q + "x": [m.width, W], q + "x.b": [m.width],
+                            q + "g": [m.width, W], q + "o": [W, m.width]})
             else:
                 out[p + "mix.q"] = [m.heads * (m.dim + m.rot_dim), W]
                 if m.kv_from is None:
@@ -357,15 +399,19 @@ class LayeredSpec:
                 out[p + "mix.uv"] = [m.heads * m.vdim, m.kv_rank]
                 out[p + "mix.g"] = [m.heads, W]
                 out[p + "mix.o"] = [W, m.heads * m.vdim]
-            if L.mlp is not None and L.mlp.kind == "dense":
+            if L.mlp is not None and L.mlp.kind == "dense" and L.mlp.act == "xielu":
+                out.update({p + "mlp.up": [L.mlp.ff, W], p + "mlp.down": [W, L.mlp.ff], p + "mlp.act": [2]})
+            elif L.mlp is not None and L.mlp.kind == "dense":
                 out.update({p + "mlp.gate": [L.mlp.ff, W], p + "mlp.up": [L.mlp.ff, W], p + "mlp.down": [W, L.mlp.ff]})
             elif L.mlp is not None:
                 for e in range(L.mlp.experts):
                     q = f"{p}mlp.e{e}."
                     out.update({q + "gate": [L.mlp.ff, W], q + "up": [L.mlp.ff, W], q + "down": [W, L.mlp.ff]})
-                out[p + "mlp.router"] = [L.mlp.experts, W]
+                out[p + "mlp.router"] = [L.mlp.experts + L.mlp.identity, W]
                 if L.mlp.router == "softmax_out":
                     out[p + "mlp.router.b"] = [L.mlp.experts]
+                if L.mlp.router == "softmax_all":
+                    out[p + "mlp.correction"] = [L.mlp.experts + L.mlp.identity]
             if self.depth_mix:
                 out[p + "dwa"] = [i + 2]
         out["final.norm"] = nshape
@@ -380,6 +426,8 @@ class LayeredSpec:
             m = self.layers[i].mixer
             if isinstance(m, LatentAttention):
                 n += m.kv_rank + m.rot_dim if m.kv_from is None else 0
+            elif isinstance(m, MinGru):
+                pass
             else:
                 a = m.attn if isinstance(m, AttentionWithRecurrence) else m
                 n += a.kv_heads * (a.dim + a.vdim)
@@ -387,8 +435,14 @@ class LayeredSpec:
 
     def state_elems(self) -> int:
         """fp32 state elements per slot (recurrent mixers), all layer runs together."""
-        return sum(self.layers[i].mixer.rec.heads * self.layers[i].mixer.rec.dim * self.layers[i].mixer.rec.vdim
-                   for i in self.runs() if isinstance(self.layers[i].mixer, AttentionWithRecurrence))
+        n = 0
+        for i in self.runs():
+            m = self.layers[i].mixer
+            if isinstance(m, AttentionWithRecurrence):
+                n += m.rec.heads * m.rec.dim * m.rec.vdim
+            elif isinstance(m, MinGru):
+                n += m.width
+        return n
 
     def step_flops(self, rows: int, ctx: int) -> float:
         """Multiply-adds x 2 of one step of `rows` tokens whose windows hold about `ctx` keys."""
@@ -396,9 +450,14 @@ class LayeredSpec:
         for i in self.runs():
             L = self.layers[i]
             m = L.mixer
+            if isinstance(m, MinGru):
+                f += 2.0 * rows * W * 4 * m.width
+                if L.mlp is not None:
+                    f += 2.0 * rows * (1 if L.mlp.kind == "dense" else L.mlp.top) * (2 if L.mlp.act == "xielu" else 3) * W * L.mlp.ff
+                continue
             if not isinstance(m, LatentAttention):
                 a = m.attn if isinstance(m, AttentionWithRecurrence) else m
-                n_in = a.heads * a.dim + a.kv_heads * (a.dim + (0 if a.values_are_keys else a.vdim))
+                n_in = a.heads * a.dim + a.kv_heads * (a.dim + (0 if a.values_are_keys else a.vdim)) + (a.heads if a.head_gate else 0)
                 n_cat = a.heads * a.vdim
                 keys = ctx if a.mask == "causal" else min(ctx, a.mask_size if a.mask == "window" else (a.mask_size + 1) // 2)
                 f += 2.0 * rows * a.heads * keys * (a.dim + a.vdim)
@@ -409,7 +468,7 @@ class LayeredSpec:
                     f += 2.0 * rows * c.heads * c.dim * c.vdim * 2
                 f += 2.0 * rows * W * (n_in + n_cat)
                 if L.mlp is not None:
-                    f += 2.0 * rows * (1 if L.mlp.kind == "dense" else L.mlp.top) * 3 * W * L.mlp.ff
+                    f += 2.0 * rows * (1 if L.mlp.kind == "dense" else L.mlp.top) * (2 if L.mlp.act == "xielu" else 3) * W * L.mlp.ff
                 continue
             n_in = m.heads * (m.dim + m.rot_dim) + m.heads + (m.kv_rank + m.rot_dim if m.kv_from is None else 0)
             f += 2.0 * rows * W * n_in + 2.0 * rows * m.heads * m.kv_rank * (m.dim + m.vdim) + 2.0 * rows * W * m.heads * m.vdim
@@ -482,7 +541,52 @@ def _nodutar_from_config(cfg: dict, name: str) -> LayeredSpec:
                        block="sandwich", tied_head=True, loop=loop)
 
 
-ARCHITECTURES = {"Tivazen": _tivazen_from_config, "Nodutar": _nodutar_from_config}
+def _lugipel_from_config(cfg: dict, name: str) -> LayeredSpec:
+    """Lugipel: pre-normed blocks (plain-weight RMS norms) over a scaled embedding with a sinusoidal
+    position vector.  Mixers: a sliding-window grouped-query attention without rotation (normed
+    queries and keys, a query temperature that grows with the position, a linear distance bias with
+    fixed head slopes, sigmoid weights with a bias per head instead of a softmax, a sigmoid gate per
+    head) or a minGRU recurrence.  Feed-forward: dense with the xIELU activation, or gated-SiLU
+    experts (some of them identity experts) routed by a softmax over all of them with a correction
+    for the choice, group-limited, renormalised and scaled.  Untied head."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m = L["mixer"]
+        if L["type"] == "attention":
+            qt = m.get("q_temp") or {}
+            mixer = GqaAttention(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]),
+                qk_norm="weight", mask="window", mask_size=int(m["mask"]["size"]), weights="sigmoid", slope_bias=True, head_gate=True,
+                q_temp_coef=float(qt.get("coef", 0.0)), q_temp_every=int(qt.get("every", 0)))
+        elif L["type"] == "mingru":
+            mixer = MinGru(width=int(m["width"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        f = L.get("mlp")
+        if f is None:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForward("dense", int(f["ff"]), act="xielu")
+        elif f["kind"] == "moe":
+            r = f["router"]
+            g = r.get("groups") or {}
+            mlp = FeedForward("moe", int(f["expert"]["ff"]), int(r["experts"]), int(r["top"]), "softmax_all",
+                              identity=int(r.get("identity", 0)), groups=int(g.get("count", 1)), groups_keep=int(g.get("keep", 1)),
+                              route_scale=float(r.get("scale", 1.0)))
+            n = mlp.experts + mlp.identity
+            if mlp.groups < 1 or n % mlp.groups or not 1 <= mlp.groups_keep <= mlp.groups:
+                raise ValueError(f"layer {i}: {n} router outputs do not form {mlp.groups} equal groups (keep {mlp.groups_keep})")
+            if mlp.top > mlp.groups_keep * (n // mlp.groups):
+                raise ValueError(f"layer {i}: top {mlp.top} above the {mlp.groups_keep} kept groups' experts")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), depth_mix=False,
+                       block="prenorm", tied_head=False, embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+                       pos_embed="sinusoid")
+
+
+ARCHITECTURES = {"Tivazen": _tivazen_from_config, "Nodutar": _nodutar_from_config, "Lugipel": _lugipel_from_config}
 
 
 def spec_from_config(cfg: dict, name: str = "model", numerics: str = "hf"):
