@@ -1477,8 +1477,8 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
         const qie_layer_desc& d = arch->layers[i];
         QIE_REQUIRE(d.ff_kind >= QIE_FF_NONE && d.ff_kind <= QIE_FF_MOE, "layer %d: unknown feed-forward %d", i, d.ff_kind);
         QIE_REQUIRE(d.ff_kind == QIE_FF_NONE || d.ff > 0, "layer %d: feed-forward size", i);
-        QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts), "layer %d: %d of %d experts", i,
-                    d.top, d.experts);
+        QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts + std::max(d.identity, 0)),
+                    "layer %d: %d of %d experts", i, d.top, d.experts + std::max(d.identity, 0));
         QIE_REQUIRE(d.router >= QIE_ROUTER_SIGMOID_IN && d.router <= QIE_ROUTER_SOFTMAX_ALL, "layer %d: router %d", i, d.router);
         QIE_REQUIRE(d.ff_act == QIE_ACT_SILU_GATED || d.ff_act == QIE_ACT_XIELU, "layer %d: activation %d", i, d.ff_act);
         if (d.ff_kind == QIE_FF_MOE && d.router == QIE_ROUTER_SOFTMAX_ALL) {

@@ -71,10 +71,9 @@ def sigmoid_attention(h, w, pre, m, eps):
         temp = query_temperature(i, m["q_temp"]["coef"], m["q_temp"]["every"])
         for hd in range(H):
             g = hd // (H // G)
-            for j in range(max(0, i - size + 1), i + 1):
-                s = float(q[i, hd] @ k[j, g]) * temp * m["scale"] - slopes[hd] * (i - j)
-                out[i, hd] += sigmoid(s + w[pre + "pb"][hd]) * v[j, g]
-            out[i, hd] *= gate[i, hd]
+            js = np.arange(max(0, i - size + 1), i + 1)          # the visible keys: 0 <= i - j < size
+            s = (k[js, g] @ q[i, hd]) * temp * m["scale"] - slopes[hd] * (i - js)
+            out[i, hd] = (sigmoid(s + w[pre + "pb"][hd]) @ v[js, g]) * gate[i, hd]
     return out.reshape(T, H * V) @ w[pre + "o"].T
 
 
@@ -106,7 +105,7 @@ def route(h_row, w, pre, r):
     """(chosen expert ids, their weights) of one row.  Experts experts .. experts + identity - 1 are
     identity experts."""
     n = r["experts"] + r["identity"]
-    z = w[pre + "router"] @ h_row
+    z = np.array([float(row @ h_row) for row in w[pre + "router"]])   # row by row: equal rows give equal logits
     s = np.exp(z - z.max())
     s = s / s.sum()
     choice = s + w[pre + "correction"]
@@ -187,6 +186,32 @@ def tensor_shapes(cfg):
     out["final.norm"] = [W]
     out["head"] = [cfg["vocab"], W]
     return out
+
+
+def attn(heads=4, kv_heads=2, dim=8, vdim=8, size=11, coef=0.3, every=4, scale=None, mlp="dense"):
+    """A layer with the attention mixer; mlp: None, "dense", a dict, or moe(...)."""
+    return {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "mask": {"size": size},
+                      "q_temp": {"coef": coef, "every": every}, "scale": float(scale if scale is not None else dim ** -0.5)},
+            "mlp": dense() if mlp == "dense" else mlp}
+
+
+def gru(width=24, mlp="dense"):
+    return {"type": "mingru", "mixer": {"width": width}, "mlp": dense() if mlp == "dense" else mlp}
+
+
+def dense(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, identity=2, top=2, count=2, keep=1, scale=1.5, ff=16):
+    return {"kind": "moe", "expert": {"ff": ff},
+            "router": {"experts": experts, "identity": identity, "top": top, "groups": {"count": count, "keep": keep}, "scale": scale}}
+
+
+def config(layers, vocab=101, width=40, eps=1e-5, embed_scale=0.5):
+    return {"architecture": "Lugipel", "vocab": vocab, "width": width, "norm": {"eps": eps}, "embedding": {"scale": embed_scale},
+            "layers": layers}
 
 
 def bf16_round(a):
