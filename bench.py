@@ -65,6 +65,15 @@ NODUTAR_SIZES = {
 }
 
 
+# Sizes of `--lugipel`: (width, heads, kv heads, head dim, window, minGRU width, dense ff, experts, identity experts,
+# top, expert groups, groups kept, expert ff, vocab).  Four layers: attention + dense xIELU, attention + routed,
+# minGRU + routed, attention + routed.
+LUGIPEL_SIZES = {
+    "1k": (1024, 16, 4, 64, 512, 2048, 2816, 8, 2, 2, 2, 1, 704, 32000),
+    "2k": (2048, 16, 4, 128, 1024, 4096, 5632, 8, 2, 2, 2, 1, 1408, 32000),
+}
+
+
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,6 +116,10 @@ def parse(argv=None):
                          "equal width / heads / ffn / layers beside it (one JSON line of its own)")
     ap.add_argument("--nodutar", choices=sorted(NODUTAR_SIZES), default=None,
                     help="instead of the default workload: prefill and decode throughput of a Nodutar model at this "
+                         "size with random weights, per-stage times, and the Qwen decoder at equal width / heads / "
+                         "layers beside it (one JSON line of its own)")
+    ap.add_argument("--lugipel", choices=sorted(LUGIPEL_SIZES), default=None,
+                    help="instead of the default workload: prefill and decode throughput of a Lugipel model at this "
                          "size with random weights, per-stage times, and the Qwen decoder at equal width / heads / "
                          "layers beside it (one JSON line of its own)")
     ap.add_argument("--dry-run", action="store_true",
@@ -166,6 +179,8 @@ def main(argv=None):
         return run_layered(a)
     if a.nodutar:
         return run_nodutar(a)
+    if a.lugipel:
+        return run_lugipel(a)
     return run(a)
 
 
@@ -217,6 +232,37 @@ def nodutar_model(S, size):
             v = np.linspace(0.1, 0.95, n, dtype=np.float32).reshape(shape)
         elif name.endswith(("r1", "r2")):
             v = np.full(shape, 0.5, np.float32)
+        else:
+            fan = shape[-1] if name != "embed" else 1
+            v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
+        tensors[name] = (np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
+    return spec, tensors
+
+
+def lugipel_model(S, size):
+    """(LayeredSpec, {name: bf16 words}) at one of LUGIPEL_SIZES, random weights from one pool."""
+    W, H, G, hd, win, gw, ff, E, ident, top, groups, keep, eff, V = LUGIPEL_SIZES[size]
+    moe = {"kind": "moe", "expert": {"ff": eff},
+           "router": {"experts": E, "identity": ident, "top": top, "groups": {"count": groups, "keep": keep}, "scale": 1.5}}
+    att = lambda mlp: {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "mask": {"size": win}, "q_temp": {"coef": 0.3, "every": 128},
+        "scale": hd ** -0.5}}
+    rec = {"type": "mingru", "mlp": moe, "mixer": {"width": gw}}
+    cfg = {"architecture": "Lugipel", "layers": [att({"kind": "dense", "ff": ff}), att(moe), rec, att(moe)], "norm": {"eps": 1e-6},
+           "embedding": {"scale": 0.5}, "vocab": V, "width": W}
+    spec = S.spec_from_config(cfg, name=f"lugipel-{size}")
+    pool = np.random.default_rng(0).standard_normal(1 << 22).astype(np.float32)
+    tensors = {}
+    for k, (name, shape) in enumerate(spec.tensor_shapes().items()):
+        n = int(np.prod(shape))
+        if name.endswith(("norm", "norm1", "norm2")):
+            v = np.ones(shape, np.float32)
+        elif name.endswith(("correction", "z.b", "x.b")):
+            v = np.zeros(shape, np.float32)
+        elif name.endswith("pb"):
+            v = np.full(shape, -4.0, np.float32)
+        elif name.endswith("act"):
+            v = np.asarray([0.5, 0.5], np.float32)
         else:
             fan = shape[-1] if name != "embed" else 1
             v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
@@ -329,6 +375,85 @@ def run_nodutar(a):
     b.close()
     eng.close()
     out["qwen_equal_size"] = qwen_twin(Q, S, Wt, a.nodutar, W, H, G, hd, 2 * top * eff, V, P, B, steps, prompts, a.prefill_iters,
+                                       max_ctx)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def run_lugipel(a):
+    """Prefill (one step of P tokens) and decode (B single-token entries a step at context ~P) of a Lugipel model,
+    per-stage hipEvent times at both shapes, and the Qwen decoder at equal sizes."""
+    import qwen_inference_engine_amd as Q
+    from qwen_inference_engine_amd import spec as S, weights as Wt
+    W, H, G, hd, win, gw, ff, E, ident, top, groups, keep, eff, V = LUGIPEL_SIZES[a.lugipel]
+    P, B, steps = a.prompt, max(a.batch, 8), min(a.steps, 128)
+    max_ctx = P + steps + 80
+    spec, tensors = lugipel_model(S, a.lugipel)
+    out = {"metric": "lugipel_decode_tokens_per_sec", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights, random token ids)", "higher_is_better": True,
+           "config": {"model": spec.name, "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "window", "mingru_width",
+                                                             "dense_ff", "experts", "identity", "top", "groups", "groups_keep",
+                                                             "expert_ff", "vocab"), LUGIPEL_SIZES[a.lugipel])),
+                      "layers": 4, "prompt": P, "decode_batch": B, "decode_steps": steps}}
+    eng = Q.Engine(spec, max_ctx=max_ctx).load_tensors(tensors)
+    del tensors
+    b = eng.batch(B, max_ctx, page_tokens=64)
+    rng = np.random.default_rng(1)
+    prompts = rng.integers(0, V, size=(B, P), dtype=np.int32)
+    ts = []
+    for it in range(1 + a.prefill_iters):
+        t0 = time.perf_counter()
+        b.step([(0, prompts[0])], [P - 1], fetch=False)
+        ts.append(time.perf_counter() - t0)
+        if it < a.prefill_iters:
+            b.release(0)
+    t_pf = float(np.median(ts[1:]))
+    stages = {"prefill": {}, "decode": {}}
+    n_in = H * hd + 2 * G * hd + H
+
+    def stage_times(tag, rows, ctx):
+        st = stages[tag]
+        st["window_attention_us"] = round(b.time_stage(1, 0, 10), 2)
+        st["attention_products_us"] = round(b.time_stage(2, 0, 10), 2)
+        st["mingru_products_us"] = round(b.time_stage(2, 2, 10), 2)
+        st["dense_ff_us"] = round(b.time_stage(3, 0, 10), 2)
+        st["routed_ff_us"] = round(b.time_stage(3, 1, 10), 2)
+        st["mingru_scan_us"] = round(b.time_stage(4, 2, 10), 2)
+        # keys a query sees: its window (a prompt's first rows see fewer)
+        kw = min(ctx, win) if tag == "decode" else (win - win * win / (2.0 * ctx) if ctx > win else ctx / 2.0)
+        st["window_attention_tflops"] = round(4.0 * rows * H * kw * hd / st["window_attention_us"] / 1e6, 2)
+        st["attention_products_tflops"] = round(2.0 * rows * W * (n_in + H * hd) / st["attention_products_us"] / 1e6, 2)
+        st["mingru_products_tflops"] = round(2.0 * rows * W * 4 * gw / st["mingru_products_us"] / 1e6, 2)
+        st["dense_ff_tflops"] = round(2.0 * rows * 2 * W * ff / st["dense_ff_us"] / 1e6, 2)
+        st["routed_ff_tflops"] = round(2.0 * rows * top * 3 * W * eff / st["routed_ff_us"] / 1e6, 2)
+        # the scan reads three projection values and writes one fp32 + one bf16 value per row and channel
+        st["mingru_scan_GBps"] = round(rows * gw * (3 * 4 + 4 + 2) / st["mingru_scan_us"] / 1e3, 1)
+        if tag == "decode":
+            st["window_attention_GBps"] = round(rows * kw * 2 * G * hd * 2 / st["window_attention_us"] / 1e3, 1)
+            st["attention_products_GBps"] = round(W * (n_in + H * hd) * 2 / st["attention_products_us"] / 1e3, 1)
+            st["mingru_products_GBps"] = round(W * 4 * gw * 2 / st["mingru_products_us"] / 1e3, 1)
+            st["dense_ff_GBps"] = round(2 * W * ff * 2 / st["dense_ff_us"] / 1e3, 1)
+        st["layer_stack_us"] = round(b.time_stage(0, 0, 5), 2)
+    stage_times("prefill", P, P)
+    b.release(0)
+    for s_ in range(B):
+        for c0 in range(0, P, 512):
+            b.step([(s_, prompts[s_][c0:c0 + 512])], [], fetch=False)
+    toks = rng.integers(0, V, size=(steps + 8, B), dtype=np.int32)
+    for i in range(8):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+    t0 = time.perf_counter()
+    for i in range(8, 8 + steps):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+        b.step_sample()
+    dt = time.perf_counter() - t0
+    stage_times("decode", B, P)
+    out.update(value=round(B * steps / dt, 1), steps=steps, warmup=8, ms_per_step=round(dt * 1e3 / steps, 4),
+               prefill_tok_s=round(P / t_pf, 1), prefill_ms=round(t_pf * 1e3, 3),
+               prefill_tflops=round(spec.step_flops(P, P // 2) / t_pf / 1e12, 2), stages=stages, vs_baseline=None)
+    b.close()
+    eng.close()
+    out["qwen_equal_size"] = qwen_twin(Q, S, Wt, a.lugipel, W, H, G, hd, 2 * top * eff, V, P, B, steps, prompts, a.prefill_iters,
                                        max_ctx)
     print(json.dumps(out), flush=True)
     return 0
