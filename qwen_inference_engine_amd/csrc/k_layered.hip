@@ -278,12 +278,25 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(const TW* E, const int3
     const int t = blockIdx.x;
     int id = tok[t];
     if (id < 0 || id >= vocab) id = 0;
-    for (int w = threadIdx.x; w < W; w += 256) {
-        float v = ldf<TW>(E, (int64_t)id * W + w) * scale;
-        if (pos) {
-            const double ang = (double)pos[t] * freq[w >> 1];
-            v += (float)((w & 1) ? cos(ang) : sin(ang));
+    if (pos) {   // a thread takes the pairs (2i, 2i + 1): one sine and cosine of the pair's angle
+        const double p = (double)pos[t];
+        for (int i = threadIdx.x; 2 * i < W; i += 256) {
+            double sn, cs;
+            sincos(p * freq[i], &sn, &cs);
+            const int w = 2 * i;
+            const float v0 = ldf<TW>(E, (int64_t)id * W + w) * scale + (float)sn;
+            out[(int64_t)t * W + w] = v0;
+            if (out_bf) out_bf[(int64_t)t * W + w] = f2bf(v0);
+            if (w + 1 < W) {
+                const float v1 = ldf<TW>(E, (int64_t)id * W + w + 1) * scale + (float)cs;
+                out[(int64_t)t * W + w + 1] = v1;
+                if (out_bf) out_bf[(int64_t)t * W + w + 1] = f2bf(v1);
+            }
         }
+        return;
+    }
+    for (int w = threadIdx.x; w < W; w += 256) {
+        const float v = ldf<TW>(E, (int64_t)id * W + w) * scale;
         out[(int64_t)t * W + w] = v;
         if (out_bf) out_bf[(int64_t)t * W + w] = f2bf(v);
     }
@@ -578,6 +591,48 @@ int xielu(const float* u, float* a, uint16_t* a_bf, int64_t n, float ap, float a
     return 0;
 }
 
+// One wave's dot product of a row y [W] (fp32) with a weight row w [W]: 8 elements per lane and turn
+// through 16-byte loads when W is a multiple of 8 (rows then start 16-byte aligned), else one
+// element per lane and turn.  The order of the sum depends on W alone.
+template <typename TW> __device__ __forceinline__ float wave_row_dot(const float* y, const TW* w, int W, int lane);
+template <> __device__ __forceinline__ float wave_row_dot<uint16_t>(const float* y, const uint16_t* w, int W, int lane) {
+    float z = 0.f;
+    if ((W & 7) == 0) {
+#pragma unroll 4
+        for (int i = lane * 8; i < W; i += 512) {
+            const uint4 u = *reinterpret_cast<const uint4*>(w + i);
+            const float4 a = *reinterpret_cast<const float4*>(y + i), b = *reinterpret_cast<const float4*>(y + i + 4);
+            z = fmaf(a.x, bf2f(u.x & 0xffffu), z);
+            z = fmaf(a.y, bf2f(u.x >> 16), z);
+            z = fmaf(a.z, bf2f(u.y & 0xffffu), z);
+            z = fmaf(a.w, bf2f(u.y >> 16), z);
+            z = fmaf(b.x, bf2f(u.z & 0xffffu), z);
+            z = fmaf(b.y, bf2f(u.z >> 16), z);
+            z = fmaf(b.z, bf2f(u.w & 0xffffu), z);
+            z = fmaf(b.w, bf2f(u.w >> 16), z);
+        }
+    } else {
+        for (int i = lane; i < W; i += 64) z = fmaf(y[i], bf2f(w[i]), z);
+    }
+    return wave_sum(z);
+}
+template <> __device__ __forceinline__ float wave_row_dot<float>(const float* y, const float* w, int W, int lane) {
+    float z = 0.f;
+    if ((W & 3) == 0) {
+#pragma unroll 4
+        for (int i = lane * 4; i < W; i += 256) {
+            const float4 a = *reinterpret_cast<const float4*>(y + i), b = *reinterpret_cast<const float4*>(w + i);
+            z = fmaf(a.x, b.x, z);
+            z = fmaf(a.y, b.y, z);
+            z = fmaf(a.z, b.z, z);
+            z = fmaf(a.w, b.w, z);
+        }
+    } else {
+        for (int i = lane; i < W; i += 64) z = fmaf(y[i], w[i], z);
+    }
+    return wave_sum(z);
+}
+
 // ------------------------------------------------------------------ mixture of experts
 // Router: z = W_r y in fp32, s = sigmoid(z); the `top` largest (ties: the lower index) in
 // descending order -> sel[t, k], score[t, k].  The ranking compares z, which orders the experts
@@ -589,9 +644,7 @@ __global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int e = wave; e < E; e += 4) {
-        float z = 0.f;
-        for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
-        z = wave_sum(z);
+        const float z = wave_row_dot<TW>(y + t * W, Wr + (int64_t)e * W, W, lane);
         if (lane == 0) s[e] = bias ? z + bias[e] : z;
     }
     __syncthreads();
@@ -649,9 +702,7 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* y, cons
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int e = wave; e < E; e += 4) {
-        float z = 0.f;
-        for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
-        z = wave_sum(z);
+        const float z = wave_row_dot<TW>(y + t * W, Wr + (int64_t)e * W, W, lane);
         if (lane == 0) s[e] = z;
     }
     __syncthreads();
