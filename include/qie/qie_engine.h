@@ -286,7 +286,7 @@ enum { QIE_BLOCK_POSTNORM_GAIN = 0, QIE_BLOCK_SANDWICH = 1, QIE_BLOCK_PRENORM = 
 enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1, QIE_ROUTER_SOFTMAX_ALL = 2 };
 /* Router 2: scores s = softmax over ALL router outputs (`experts` experts with weights, then
  * `identity` experts whose output is their input); experts are chosen by s + correction ('l<i>.mlp.
- * correction'), only inside the `groups_keep` best of `groups` equal groups of neighbouring
+ * correction'), only inside the `groups_keep` best of `groups` contiguous, equally sized groups of
  * outputs (a group's rank: its largest s + correction); the `top` chosen are weighted by
  * s / (sum of the chosen s + 1e-20) * route_scale, applied to the experts' outputs. */
 /* Dense feed-forward: 0 = W_down (silu(W_gate h) * W_up h); 1 = W_down xielu(W_up h) with the two
@@ -294,7 +294,7 @@ enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1, QIE_ROUTER_SOFTMAX
  * (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.  Experts are always of form 0. */
 enum { QIE_ACT_SILU_GATED = 0, QIE_ACT_XIELU = 1 };
 /* Attention weights of the visible keys: softmax of the scores, or sigmoid(score + pb_h) with a
- * number per head ('mix.pb'), not normalised over the keys. */
+ * number per head ('mix.pb'); a row's weights are used as they are. */
 enum { QIE_WEIGHTS_SOFTMAX = 0, QIE_WEIGHTS_SIGMOID = 1 };
 /* Positions in the embedding: none, or the vector with entry 2i = sin(p * 10000^(-2i / width)),
  * entry 2i + 1 = cos of the same, added to the scaled embedding row. */
@@ -338,7 +338,7 @@ typedef struct qie_recurrent_desc {
     int32_t reserved;
 } qie_recurrent_desc;
 
-/* Mixer QIE_MIXER_MINGRU: a gated recurrence whose gates read only the current token.  With x the
+/* Mixer QIE_MIXER_MINGRU: a recurrence per channel whose update gate and candidate depend on the current input alone.  With x the
  * mixer's input: z = sigmoid(W_z x + b_z), u = W_x x + b_x (`width` channels each), candidate
  * c = u + 1/2 where u >= 0, sigmoid(u) where u < 0; per channel S_t = (1 - z_t) S_(t-1) + z_t c_t,
  * S fp32 in the slot, zero at position 0; output W_o (S_t * silu(W_g x)).  Tensors

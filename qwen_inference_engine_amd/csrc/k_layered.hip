@@ -689,7 +689,7 @@ int route_topk(const float* y, const void* Wr, const float* bias, bool w_f32, in
 
 // Router over all E outputs (real and identity experts alike): s = softmax(z) in fp32; the choice
 // ranks s + corr; a group of E / groups neighbours ranks by its largest choice score and only the
-// `keep` best groups stay eligible (the others count as minus infinity); the `top` best eligible
+// `keep` best groups stay eligible (the others are excluded from the choice); the `top` best eligible
 // are chosen, weighted by s / (sum of the chosen s + 1e-20) * scale.  Ties: the lower index.
 // One block per row; shared: s [E], choice [E], group rank [groups].
 template <typename TW>

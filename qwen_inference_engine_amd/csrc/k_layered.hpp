@@ -162,7 +162,7 @@ struct GqaAttnP {
     int out_col;
     const float* slopes;      // [heads] or null: the score also loses slopes[h] * (i - j)
     const float* pb;          // [heads] or null; set: a visible key's weight is sigmoid(score + pb[h]),
-                              // not normalised over the keys (no softmax)
+                              // and the weights of a row are used as they are (no softmax)
     int gate_col;             // >= 0: head h's result times sigmoid(proj[t * ld + gate_col + h])
 };
 int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);

@@ -8,7 +8,7 @@
 //                        and / or a linear one with a slope per head; softmax weights, or sigmoid
 //                        weights with a bias per head; an optional sigmoid gate per head
 //   lay::gated_scan      gated linear recurrence with an fp32 state per slot and head
-//   lay::mingru_scan     minGRU: a gated recurrence per channel whose gates read the current token
+//   lay::mingru_scan     minGRU: a recurrence per channel, update gate and candidate from the current input alone
 //   lay::head_norm_rows  per-head RMS norm with a weight
 //   lay::add_norm        residual add of a normed branch fused with the next branch's input norm
 //

@@ -230,7 +230,7 @@ class AttentionWithRecurrence:
 
 @dataclasses.dataclass(frozen=True)
 class MinGru:
-    """Mixer: minGRU, a gated recurrence whose gates read only the current token; `width` fp32 state
+    """Mixer: minGRU, a recurrence per channel whose update gate and candidate depend on the current input alone; `width` fp32 state
     elements per slot."""
     width: int
 

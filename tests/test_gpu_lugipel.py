@@ -200,7 +200,7 @@ def test_xielu_both_branches_and_its_two_numbers(model):
 
 def test_router_correction_groups_and_negative_choice_scores(model):
     """A correction far below zero makes every choice score negative: the experts outside the kept group must
-    count as minus infinity, not zero; the correction picks the experts but the weights are the plain scores."""
+    be excluded outright (a masked score of zero would win against them); the correction picks the experts but the weights are the plain scores."""
     def tw(T, cfg):
         T["l0.mlp.correction"][:] = np.array([-5.0, -6.25, -7.5, -3.0, -6.0, -6.5, -7.0, -4.5], dtype=np.float32)
     m = model([gru(mlp=moe(6, 2, 2, 2, 1, 1.5))], seed=6, tweak=tw)
@@ -372,6 +372,8 @@ def test_long_portions_run_the_recurrence_in_pieces(model):
     (8, 2, 64, 32, 64, 200),
     (2, 1, 128, 64, 32, 33),     # head ratio 2: heads packed into a wave's columns
     (3, 3, 32, 128, 64, 90),
+    (8, 1, 32, 32, 32, 70),      # eight heads of one key head: two workgroups share its tiles
+    (6, 2, 64, 32, 64, 45),      # head ratio 3: packed
     (4, 4, 64, 64, 16, 40),      # pages too small for the matrix-core form: the plain kernel on bf16 rows
 ])
 def test_bf16_attention_shapes(model, heads, kv, dim, vdim, pt, size):
