@@ -266,7 +266,8 @@ int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_id
  * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains; each branch is
  * normed after it is computed, its input is the raw stream); the next layer's input is the depth-weighted sum over the embedding
  * output and every layer result so far. */
-enum { QIE_MIXER_LATENT_ATTENTION = 1, QIE_MIXER_GQA = 2, QIE_MIXER_GQA_RECURRENT = 3, QIE_MIXER_MINGRU = 4 };
+enum { QIE_MIXER_LATENT_ATTENTION = 1, QIE_MIXER_GQA = 2, QIE_MIXER_GQA_RECURRENT = 3, QIE_MIXER_MINGRU = 4,
+       QIE_MIXER_CHANNEL_DELTA = 5 };
 enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
 /* Which keys j <= i a query at position i sees: all of them; the last `size`; those of its own
  * block of `size` positions (blocks counted from position 0 of the sequence). */
@@ -278,8 +279,11 @@ enum { QIE_QKNORM_NONE = 0, QIE_QKNORM_WEIGHT = 1, QIE_QKNORM_PLAIN = 2 };
 enum { QIE_ROT_HALVES = 0, QIE_ROT_INTERLEAVED = 1 };
 /* Block: 0 = y = x + g * rms(branch(x)) with scalar gains (branches read the raw stream);
  * 1 = x += N_b(branch(N_a(x))) with weight vectors stored around zero (N(v) = rms(v) (1 + w))
- * before and after every branch; 2 = x += branch(N(x)) with N(v) = rms(v) w (plain weight vectors
- * 'l<i>.norm1|norm2', 'final.norm'), one norm before every branch and none after. */
+ * before and after every branch; 2 = x += branch(N(x)) with N(v) = rms(v) (norm_offset + w) (weight
+ * vectors 'l<i>.norm1|norm2', 'final.norm'; norm_offset 0: plain weights, 1: stored around zero), one
+ * norm before every branch and none after.  Options of block 2 (qie_arch_desc): several residual
+ * streams with learned mixing (streams), a causal convolution on the mixer's normed input
+ * (canon_taps), a norm of the embedding rows (embed_norm). */
 enum { QIE_BLOCK_POSTNORM_GAIN = 0, QIE_BLOCK_SANDWICH = 1, QIE_BLOCK_PRENORM = 2 };
 /* Router: 0 = sigmoid scores, the `top` largest scale the experts' input; 1 = logits with a
  * bias, the `top` largest weighted by the softmax over those alone scale the experts' output. */
@@ -292,7 +296,8 @@ enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1, QIE_ROUTER_SOFTMAX
 /* Dense feed-forward: 0 = W_down (silu(W_gate h) * W_up h); 1 = W_down xielu(W_up h) with the two
  * numbers p, q of 'l<i>.mlp.act': xielu(z) = softplus(p) z^2 + z / 2 for z > 0, else
  * (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.  Experts are always of form 0. */
-enum { QIE_ACT_SILU_GATED = 0, QIE_ACT_XIELU = 1 };
+/* 2 = W_down (gelu_tanh(W_gate h) * W_up h), gelu_tanh(z) = z / 2 (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))). */
+enum { QIE_ACT_SILU_GATED = 0, QIE_ACT_XIELU = 1, QIE_ACT_GELU_TANH_GATED = 2 };
 /* Attention weights of the visible keys: softmax of the scores, or sigmoid(score + pb_h) with a
  * number per head ('mix.pb'); a row's weights are used as they are. */
 enum { QIE_WEIGHTS_SOFTMAX = 0, QIE_WEIGHTS_SIGMOID = 1 };
@@ -308,6 +313,13 @@ enum { QIE_POS_NONE = 0, QIE_POS_SINUSOID = 1 };
  * angle j * rot_base^(-2m / vdim)), cached so, and a head's weighted sum at position i is turned
  * back by i; the mask; values_are_keys: no W_v, the value is the projected key as it leaves W_k
  * (before its norm; vdim == dim); dist_bias: the score loses r1_h * ln(1 + r2_h * (i - j)). */
+/* Rotary frequencies scaled by their wavelength l = 2 pi / f (factor 0: no scaling): f stays where
+ * l < original / high, becomes f / factor where l > original / low, and between the two, with
+ * s = (original / l - low) / (high - low), (1 - s) f / factor + s f. */
+typedef struct qie_rot_scaling {
+    float factor, low, high, original;
+} qie_rot_scaling;
+
 typedef struct qie_gqa_desc {
     int32_t heads, kv_heads, dim, vdim;
     int32_t qk_norm;          /* QIE_QKNORM_*   */
@@ -318,13 +330,19 @@ typedef struct qie_gqa_desc {
     int32_t values_are_keys;
     int32_t dist_bias;
     float rot_base, scale;
-    int32_t reserved[2];
+    int32_t qk_bias;          /* 1: q and k get a bias vector after their projection ('mix.q.b', 'mix.k.b'); a key cached as
+                                 the value carries its bias */
+    int32_t sink;             /* 1: the softmax denominator also holds exp(sink_h), a number per head ('mix.sink') that has
+                                 no key and no value                                                             */
     int32_t weights;          /* QIE_WEIGHTS_*                                               */
     int32_t slope_bias;       /* 1: the score loses 2^(-8 (h + 1) / heads) * (i - j)         */
     int32_t head_gate;        /* 1: head h's output times sigmoid(W_g x)_h ('mix.g' [heads, width]) */
     int32_t q_temp_every;     /* > 0: after its norm q is multiplied by                      */
     float q_temp_coef;        /*   1 + coef * ln(floor((pos + 1) / every) + 1)               */
-    int32_t reserved2[3];
+    int32_t out_gate;         /* 1: the concatenated head outputs times sigmoid(W_g x), element by element
+                                 ('mix.g' [heads * vdim, width])                             */
+    int32_t reserved2[2];
+    qie_rot_scaling rot_scaling;
 } qie_gqa_desc;
 
 /* Gated linear recurrence (the second half of QIE_MIXER_GQA_RECURRENT): per head a state
@@ -348,6 +366,21 @@ typedef struct qie_mingru_desc {
     int32_t reserved[3];
 } qie_mingru_desc;
 
+/* Mixer QIE_MIXER_CHANNEL_DELTA: gated delta rule with one decay per head and key channel.  With x the
+ * mixer's input: q = W_q x, k = W_k x (kv_heads x dim), v = W_v x (heads x vdim); each passes a causal
+ * convolution over time per channel ('mix.q.conv' etc. [channels, conv], last column = the current
+ * token) and silu; q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q times dim^(-1/2);
+ * beta = sigmoid(W_b x) per head; decay g = exp(-exp(A_log_h) softplus(W_a2 (W_a1 x) + dt_bias)), heads x
+ * dim.  Per head (query / key head h / (heads / kv_heads)), S [dim][vdim] fp32 in the slot, zero at
+ * position 0: S = diag(g) S; u = beta (v - S^T k); S += k u^T; o = S^T q.  o is RMS-normed per head over
+ * vdim with the weight 'mix.norm' [vdim], times sigmoid(W_g2 (W_g1 x)) (heads x vdim), then W_o.  The
+ * last conv - 1 rows of q, k, v before their convolution belong to the slot's state.  rank_a / rank_g:
+ * rows of W_a1 / W_g1.  Tensors 'l<i>.mix.q|q.conv|k|k.conv|v|v.conv|b|A_log|a1|a2|dt_bias|g1|g2|norm|o'. */
+typedef struct qie_delta_desc {
+    int32_t heads, kv_heads, dim, vdim, conv, rank_a, rank_g;
+    int32_t reserved;
+} qie_delta_desc;
+
 typedef struct qie_layer_desc {
     int32_t mixer;            /* QIE_MIXER_*                                          */
     int32_t heads, dim, rot_dim, vdim, kv_rank;
@@ -359,7 +392,10 @@ typedef struct qie_layer_desc {
     int32_t ff;               /* hidden size of the dense feed-forward / of one expert */
     int32_t experts, top;
     int32_t router;           /* QIE_ROUTER_*                                          */
-    int32_t reserved[3];
+    /* latent attention options: q_rank > 0: the queries come through a latent of their own,
+     * q = W_uq rms(W_dq x) w ('mix.dq' [q_rank, width], 'mix.dq.norm', 'mix.uq'; no 'mix.q');
+     * rot_layout QIE_ROT_*; head_gate 1: the per-head sigmoid gate 'mix.g'.  window 0: every j <= i. */
+    int32_t q_rank, rot_layout, head_gate;
     qie_gqa_desc gqa;         /* QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT                */
     qie_recurrent_desc rec;   /* QIE_MIXER_GQA_RECURRENT                               */
     float gqa_scale, rec_scale;
@@ -369,6 +405,8 @@ typedef struct qie_layer_desc {
     int32_t groups, groups_keep;
     float route_scale;
     int32_t reserved3[3];
+    qie_delta_desc delta;     /* QIE_MIXER_CHANNEL_DELTA                               */
+    qie_rot_scaling rot_scaling;   /* latent attention                                 */
 } qie_layer_desc;
 
 typedef struct qie_arch_desc {
@@ -384,6 +422,16 @@ typedef struct qie_arch_desc {
     int32_t pos_embed;        /* QIE_POS_*                                              */
     float embed_scale;        /* the embedding row is multiplied by it (0 is read as 1) */
     const qie_layer_desc* layers;
+    /* QIE_BLOCK_PRENORM only.  streams >= 1: `streams` copies x_1 .. x_n of the residual row, all equal to
+     * the embedding output at the start; sublayer q of layer i (1 mixer, 2 feed-forward) reads
+     * u = sum_s in[s] x_s, computes y = sublayer(N(u)) and sets, all at once from the old rows,
+     * x_t = sum_s mix[s][t] x_s + out[t] y ('l<i>.hc<q>.in|out' [streams], 'l<i>.hc<q>.mix' [streams,
+     * streams]); the output norm reads the sum of the rows.  0: one row, x += y.
+     * canon_taps >= 1: the mixer reads h + conv(h) instead of its normed input h, conv(h)_t = sum_j w[:, j]
+     * h_(t - taps + 1 + j) per channel ('l<i>.canon1' [width, taps]); the last taps - 1 rows h belong to
+     * the slot's state.  embed_norm 1: the embedding rows pass N with 'embed.norm' first. */
+    int32_t streams, canon_taps, embed_norm;
+    float norm_offset;
 } qie_arch_desc;
 
 int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* opts, qie_engine** out);
@@ -393,6 +441,8 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
  * attention), 'l<i>.mix.q|k|v|q.norm|k.norm|r1|r2|o' (QIE_MIXER_GQA; under 'l<i>.mix.left.' when a
  * recurrence runs beside it, whose tensors are 'l<i>.mix.right.q|f|f.b|lower|v|norm|o'),
  * 'l<i>.mix.pb|g' (sigmoid weights, head gate), 'l<i>.mix.z|z.b|x|x.b|g|o' (QIE_MIXER_MINGRU),
+ * 'l<i>.mix.q.b|k.b|sink' (biased, sink attention), 'l<i>.mix.dq|dq.norm|uq' (latent queries), the
+ * QIE_MIXER_CHANNEL_DELTA tensors, 'embed.norm', 'l<i>.hc1|hc2.in|out|mix', 'l<i>.canon1',
  * 'l<i>.mlp.gate|up|down|act|router|router.b|correction', 'l<i>.mlp.e<j>.gate|up|down'.
  * qie_engine_finalize_weights checks every tensor the architecture needs against its shape,
  * builds the device layouts (fused projection rows, per-head transposed W_uk, experts end to
@@ -426,8 +476,8 @@ int qie_batch_keep_layers(qie_batch* b, int32_t enable);
 int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n);
 /* Time `iters` runs of one stage of the last step's shape (hipEvents on the engine stream):
  * which 0 = the whole layer stack, 1 = attention of `layer`, 2 = its projections (input, absorb,
- * value expansion, output), 3 = its feed-forward, 4 = its recurrence (gated scan + head norm, or the
- * minGRU scan; the slots' states of that layer run are advanced by it, so time it last).  The cache is read, not
+ * value expansion, output), 3 = its feed-forward, 4 = its recurrence (gated scan + head norm, the
+ * minGRU scan, or the delta rule's gates, scan and output norm; the slots' states of that layer run are advanced by it, so time it last).  The cache is read, not
  * advanced. */
 int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us);
 

@@ -81,25 +81,29 @@ class EngineOptsC(C.Structure):
                 ("compute_f32", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
-QIE_MIXER_LATENT_ATTENTION, QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT, QIE_MIXER_MINGRU = 1, 2, 3, 4
+QIE_MIXER_LATENT_ATTENTION, QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT, QIE_MIXER_MINGRU, QIE_MIXER_CHANNEL_DELTA = 1, 2, 3, 4, 5
 QIE_FF_NONE, QIE_FF_DENSE, QIE_FF_MOE = 0, 1, 2
 QIE_MASK_CAUSAL, QIE_MASK_WINDOW, QIE_MASK_CHUNK = 0, 1, 2
 QIE_QKNORM_NONE, QIE_QKNORM_WEIGHT, QIE_QKNORM_PLAIN = 0, 1, 2
 QIE_ROT_HALVES, QIE_ROT_INTERLEAVED = 0, 1
 QIE_BLOCK_POSTNORM_GAIN, QIE_BLOCK_SANDWICH, QIE_BLOCK_PRENORM = 0, 1, 2
 QIE_ROUTER_SIGMOID_IN, QIE_ROUTER_SOFTMAX_OUT, QIE_ROUTER_SOFTMAX_ALL = 0, 1, 2
-QIE_ACT_SILU_GATED, QIE_ACT_XIELU = 0, 1
+QIE_ACT_SILU_GATED, QIE_ACT_XIELU, QIE_ACT_GELU_TANH_GATED = 0, 1, 2
 QIE_WEIGHTS_SOFTMAX, QIE_WEIGHTS_SIGMOID = 0, 1
 QIE_POS_NONE, QIE_POS_SINUSOID = 0, 1
+
+
+class RotScalingC(C.Structure):
+    _fields_ = [("factor", C.c_float), ("low", C.c_float), ("high", C.c_float), ("original", C.c_float)]
 
 
 class GqaDescC(C.Structure):
     _fields_ = [("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32),
                 ("qk_norm", C.c_int32), ("rot_dims", C.c_int32), ("rot_layout", C.c_int32), ("rot_values", C.c_int32),
                 ("mask", C.c_int32), ("mask_size", C.c_int32), ("values_are_keys", C.c_int32), ("dist_bias", C.c_int32),
-                ("rot_base", C.c_float), ("scale", C.c_float), ("reserved", C.c_int32 * 2),
+                ("rot_base", C.c_float), ("scale", C.c_float), ("qk_bias", C.c_int32), ("sink", C.c_int32),
                 ("weights", C.c_int32), ("slope_bias", C.c_int32), ("head_gate", C.c_int32), ("q_temp_every", C.c_int32),
-                ("q_temp_coef", C.c_float), ("reserved2", C.c_int32 * 3)]
+                ("q_temp_coef", C.c_float), ("out_gate", C.c_int32), ("reserved2", C.c_int32 * 2), ("rot_scaling", RotScalingC)]
 
 
 class RecurrentDescC(C.Structure):
@@ -110,22 +114,29 @@ class MinGruDescC(C.Structure):
     _fields_ = [("width", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
+class DeltaDescC(C.Structure):
+    _fields_ = [("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32), ("conv", C.c_int32),
+                ("rank_a", C.c_int32), ("rank_g", C.c_int32), ("reserved", C.c_int32)]
+
+
 class LayerDescC(C.Structure):
     _fields_ = [("mixer", C.c_int32), ("heads", C.c_int32), ("dim", C.c_int32), ("rot_dim", C.c_int32),
                 ("vdim", C.c_int32), ("kv_rank", C.c_int32), ("window", C.c_int32), ("kv_from", C.c_int32),
                 ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("scale", C.c_float),
                 ("ff_kind", C.c_int32), ("ff", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
-                ("router", C.c_int32), ("reserved", C.c_int32 * 3),
+                ("router", C.c_int32), ("q_rank", C.c_int32), ("rot_layout", C.c_int32), ("head_gate", C.c_int32),
                 ("gqa", GqaDescC), ("rec", RecurrentDescC), ("gqa_scale", C.c_float), ("rec_scale", C.c_float),
                 ("mingru", MinGruDescC), ("ff_act", C.c_int32), ("identity", C.c_int32), ("groups", C.c_int32),
-                ("groups_keep", C.c_int32), ("route_scale", C.c_float), ("reserved3", C.c_int32 * 3)]
+                ("groups_keep", C.c_int32), ("route_scale", C.c_float), ("reserved3", C.c_int32 * 3),
+                ("delta", DeltaDescC), ("rot_scaling", RotScalingC)]
 
 
 class ArchDescC(C.Structure):
     _fields_ = [("n_layers", C.c_int32), ("width", C.c_int32), ("vocab", C.c_int32), ("norm_eps", C.c_float),
                 ("depth_mix", C.c_int32), ("block", C.c_int32), ("tied_head", C.c_int32),
                 ("loop_start", C.c_int32), ("loop_stop", C.c_int32), ("loop_times", C.c_int32),
-                ("pos_embed", C.c_int32), ("embed_scale", C.c_float), ("layers", C.POINTER(LayerDescC))]
+                ("pos_embed", C.c_int32), ("embed_scale", C.c_float), ("layers", C.POINTER(LayerDescC)),
+                ("streams", C.c_int32), ("canon_taps", C.c_int32), ("embed_norm", C.c_int32), ("norm_offset", C.c_float)]
 
 
 # (name, restype, argtypes) — every symbol the public headers declare.

@@ -37,6 +37,7 @@ struct HostTensor {
 struct RopeTab {
     double base;
     int dims;
+    qie_rot_scaling sc;   // factor 0: unscaled frequencies
     float* cs;
     float* sn;
 };
@@ -74,6 +75,21 @@ struct LayerDev {
     // xIELU: softplus(p), 1/2 + softplus(q); the grouped router's correction
     float act_p = 0.f, act_q = 0.f;
     float* correction = nullptr;
+    // attention options: bias vectors of q and k, the softmax sink per head
+    float *q_bias = nullptr, *k_bias = nullptr, *sink = nullptr;
+    // latent queries through a latent of their own: w_in = [dq ; (dkv)] rows (n_pre of them), the
+    // latent's norm weight, W_uq [heads * (dim + rot_dim)][q_rank]
+    void* w_uq = nullptr;
+    float* dq_norm = nullptr;
+    int n_pre = 0;
+    // hyper-connections of sublayer 1 (mixer) and 2 (feed-forward); the input convolution's taps [width][taps]
+    float *hc_in[2] = {nullptr, nullptr}, *hc_out[2] = {nullptr, nullptr}, *hc_mix[2] = {nullptr, nullptr};
+    float* canon = nullptr;
+    // QIE_MIXER_CHANNEL_DELTA: w_in = [q ; k ; v ; b ; a1 ; g1] rows, W_a2, W_g2, the three short
+    // convolutions' taps end to end [2 G dim + H vdim][conv], exp(A_log), dt_bias, the head norm's weight
+    void *w_a2 = nullptr, *w_g2 = nullptr;
+    float *dl_conv = nullptr, *dl_exp_a = nullptr, *dl_dt_bias = nullptr, *dl_norm = nullptr;
+    int col_b = 0, col_a1 = 0, col_g1 = 0, rank_a = 0, rank_g = 0;
 };
 
 // One execution of a layer: layers of a repeated group run several times, each run with its
@@ -94,6 +110,7 @@ struct LayeredModel {
     void* head = nullptr;
     float g_final = 1.f;
     float* w_final = nullptr;   // sandwich and pre-norm blocks: the output norm's weight vector
+    float* w_embed = nullptr;   // the embedding rows' norm (embed_norm)
     double* pos_freq = nullptr; // sinusoidal positions: 10000^(-2i / width), i < ceil(width / 2)
     std::vector<LayerRun> runs;
     bool loops = false;
@@ -106,6 +123,11 @@ struct LayeredBatch {
     std::vector<int64_t> layer_off;   // per layer run: element offset of its (K) rows inside a page
     std::vector<int64_t> v_off;       // per layer run: its V rows (grouped-query attention)
     std::vector<int64_t> state_off;   // per layer run: its recurrent state inside a slot's state
+    std::vector<int64_t> conv_off;    // per layer run: the last inputs of its short convolutions (delta rule)
+    std::vector<int64_t> canon_off;   // per layer run: the last normed mixer inputs (input convolution)
+    float *pre = nullptr, *aux = nullptr;   // first-stage projections / convolved q, k, v; second-stage gate logits
+    int64_t m_pre = 0, m_aux = 0;
+    int32_t* row_k = nullptr;         // a row's index inside its entry
     float* state = nullptr;           // [slots][slot_state] fp32
     int64_t slot_state = 0;
     int4* d_ent = nullptr;            // the step's entries {first packed row, rows, slot, first position}
@@ -244,22 +266,33 @@ static int lm_floats(LayeredModel* m, float** dev, const HostTensor& t) {
     return 0;
 }
 
-static int lm_rope(LayeredModel* m, qie_engine* e, double base, int dims, int* index) {
+static int lm_rope(LayeredModel* m, qie_engine* e, double base, int dims, int* index, const qie_rot_scaling* scp = nullptr) {
+    qie_rot_scaling sc{};
+    if (scp && scp->factor > 0.f) sc = *scp;
     for (size_t i = 0; i < m->ropes.size(); i++)
-        if (m->ropes[i].base == base && m->ropes[i].dims == dims) {
+        if (m->ropes[i].base == base && m->ropes[i].dims == dims && memcmp(&m->ropes[i].sc, &sc, sizeof(sc)) == 0) {
             *index = (int)i;
             return 0;
         }
     const int half = dims / 2, rows = e->opts.max_ctx;
     std::vector<float> cs((size_t)rows * half), sn((size_t)rows * half);
     for (int j = 0; j < half; j++) {
-        const double f = std::pow(base, -2.0 * j / dims);
+        double f = std::pow(base, -2.0 * j / dims);
+        if (sc.factor > 0.f) {   // by wavelength: short ones stay, long ones slow down by the factor, a blend between
+            const double lam = 2.0 * M_PI / f, orig = sc.original;
+            if (lam > orig / sc.low)
+                f = f / sc.factor;
+            else if (lam >= orig / sc.high) {
+                const double t = (orig / lam - sc.low) / ((double)sc.high - sc.low);
+                f = (1.0 - t) * f / sc.factor + t * f;
+            }
+        }
         for (int p = 0; p < rows; p++) {
             cs[(size_t)p * half + j] = (float)std::cos(p * f);
             sn[(size_t)p * half + j] = (float)std::sin(p * f);
         }
     }
-    RopeTab t{base, dims, nullptr, nullptr};
+    RopeTab t{base, dims, sc, nullptr, nullptr};
     QIE_TRY(lm_alloc(m, (void**)&t.cs, cs.size() * 4 + 16));
     QIE_TRY(lm_alloc(m, (void**)&t.sn, sn.size() * 4 + 16));
     QIE_HIP(hipMemcpy(t.cs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
@@ -300,8 +333,8 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
     const int64_t rq = rec ? (int64_t)d.rec.heads * d.rec.dim : 0, rv = rec ? (int64_t)d.rec.heads * d.rec.vdim : 0;
     L.col_k = (int)nq;
     L.col_v = a.values_are_keys ? -1 : (int)(nq + nk);
-    const int64_t ng = a.head_gate ? a.heads : 0;
-    L.col_gate = a.head_gate ? (int)(nq + nk + nv) : -1;
+    const int64_t ng = a.out_gate ? (int64_t)a.heads * a.vdim : a.head_gate ? a.heads : 0;
+    L.col_gate = ng ? (int)(nq + nk + nv) : -1;
     L.col_rq = (int)(nq + nk + nv + ng);
     L.col_rf = (int)(L.col_rq + rq);
     L.col_rv = (int)(L.col_rf + rq);
@@ -323,10 +356,15 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
         QIE_TRY(lm_vector(m, &L.r1, pa + "r1", a.heads));
         QIE_TRY(lm_vector(m, &L.r2, pa + "r2", a.heads));
     }
-    if (a.head_gate) {
-        LM_GET(tg, pa + "g", (int64_t)a.heads, W);
+    if (ng) {
+        LM_GET(tg, pa + "g", ng, W);
         QIE_TRY(lm_upload_rows(m, L.w_in, L.col_gate, W, *tg));
     }
+    if (a.qk_bias) {
+        QIE_TRY(lm_vector(m, &L.q_bias, pa + "q.b", nq));
+        QIE_TRY(lm_vector(m, &L.k_bias, pa + "k.b", nk));
+    }
+    if (a.sink) QIE_TRY(lm_vector(m, &L.sink, pa + "sink", a.heads));
     if (a.weights == QIE_WEIGHTS_SIGMOID) QIE_TRY(lm_vector(m, &L.pb, pa + "pb", a.heads));
     if (a.slope_bias) {
         HostTensor sl;
@@ -336,7 +374,7 @@ static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
         for (int h = 0; h < a.heads; h++) ((float*)sl.data.data())[h] = (float)std::exp2(-8.0 * (h + 1) / a.heads);
         QIE_TRY(lm_floats(m, &L.slopes, sl));
     }
-    if (a.rot_dims > 0) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.rot_dims, &L.rope));
+    if (a.rot_dims > 0) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.rot_dims, &L.rope, &a.rot_scaling));
     if (a.rot_values) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.vdim, &L.rope_v));
     const int64_t ca = (int64_t)a.heads * a.vdim;
     L.cat_rec = (int)ca;
@@ -396,10 +434,95 @@ static int finalize_mingru(LayeredModel* m, int i) {
     return 0;
 }
 
+// Gated delta rule: fused input rows [q ; k ; v ; b ; a1 ; g1], the second-stage matrices, the three
+// convolutions' taps end to end, exp(A_log) in double.  rank_a / rank_g 0: the rows of 'a1' / 'g1'.
+static int finalize_delta(LayeredModel* m, int i) {
+    LayerDev& L = m->L[i];
+    const qie_delta_desc& c = L.d.delta;
+    const int64_t W = m->a.width, nk = (int64_t)c.kv_heads * c.dim, nv = (int64_t)c.heads * c.vdim, C = 2 * nk + nv;
+    const std::string px = "l" + std::to_string(i) + ".mix.";
+    auto rows_of = [&](const std::string& name) -> int64_t {
+        auto it = m->host.find(name);
+        return it != m->host.end() && it->second.shape.size() == 2 ? it->second.shape[0] : 0;
+    };
+    L.rank_a = c.rank_a > 0 ? c.rank_a : (int)rows_of(px + "a1");
+    L.rank_g = c.rank_g > 0 ? c.rank_g : (int)rows_of(px + "g1");
+    QIE_REQUIRE(L.rank_a > 0 && L.rank_g > 0, "layered weights: layer %d: tensors '%sa1' / '%sg1' give no rank", i, px.c_str(), px.c_str());
+    L.col_k = (int)nk;
+    L.col_v = (int)(2 * nk);
+    L.col_b = (int)C;
+    L.col_a1 = (int)(C + c.heads);
+    L.col_g1 = L.col_a1 + L.rank_a;
+    L.n_in = L.col_g1 + L.rank_g;
+    L.n_cat = (int)nv;
+    QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
+    LM_GET(tq, px + "q", nk, W);
+    LM_GET(tk, px + "k", nk, W);
+    LM_GET(tv, px + "v", nv, W);
+    LM_GET(tb, px + "b", (int64_t)c.heads, W);
+    LM_GET(ta1, px + "a1", (int64_t)L.rank_a, W);
+    LM_GET(tg1, px + "g1", (int64_t)L.rank_g, W);
+    QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tq));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_k, W, *tk));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_v, W, *tv));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_b, W, *tb));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_a1, W, *ta1));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_g1, W, *tg1));
+    LM_GET(ta2, px + "a2", (int64_t)c.heads * c.dim, (int64_t)L.rank_a);
+    LM_GET(tg2, px + "g2", nv, (int64_t)L.rank_g);
+    QIE_TRY(lm_alloc(m, &L.w_a2, (size_t)ta2->numel() * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.w_a2, 0, L.rank_a, *ta2));
+    QIE_TRY(lm_alloc(m, &L.w_g2, (size_t)tg2->numel() * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.w_g2, 0, L.rank_g, *tg2));
+    LM_GET(cq, px + "q.conv", nk, (int64_t)c.conv);
+    LM_GET(ck, px + "k.conv", nk, (int64_t)c.conv);
+    LM_GET(cv, px + "v.conv", nv, (int64_t)c.conv);
+    {
+        HostTensor cat;
+        cat.dtype = 2;
+        cat.shape = {C, (int64_t)c.conv};
+        cat.data.resize((size_t)C * c.conv * 4);
+        float* f = (float*)cat.data.data();
+        int64_t o = 0;
+        for (const HostTensor* t : {cq, ck, cv})
+            for (int64_t k = 0; k < t->numel(); k++) f[o++] = host_elem(*t, k);
+        QIE_TRY(lm_floats(m, &L.dl_conv, cat));
+    }
+    LM_GET(tal, px + "A_log", (int64_t)c.heads);
+    {
+        HostTensor ea;
+        ea.dtype = 2;
+        ea.shape = {(int64_t)c.heads};
+        ea.data.resize((size_t)c.heads * 4);
+        for (int h = 0; h < c.heads; h++) ((float*)ea.data.data())[h] = (float)std::exp((double)host_elem(*tal, h));
+        QIE_TRY(lm_floats(m, &L.dl_exp_a, ea));
+    }
+    QIE_TRY(lm_vector(m, &L.dl_dt_bias, px + "dt_bias", (int64_t)c.heads * c.dim));
+    QIE_TRY(lm_vector(m, &L.dl_norm, px + "norm", (int64_t)c.vdim));
+    LM_GET(to, px + "o", W, nv);
+    QIE_TRY(lm_alloc(m, &L.wo, (size_t)W * nv * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.wo, 0, nv, *to));
+    return 0;
+}
+
 static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
     LayerDev& L = m->L[i];
     const qie_layer_desc& d = L.d;
     const std::string pl = "l" + std::to_string(i) + ".", px = pl + "mix.";
+    if (m->a.streams > 0) {
+        const int64_t n = m->a.streams;
+        for (int q = 0; q < (d.ff_kind != QIE_FF_NONE ? 2 : 1); q++) {
+            const std::string ph = pl + "hc" + std::to_string(q + 1) + ".";
+            QIE_TRY(lm_vector(m, &L.hc_in[q], ph + "in", n));
+            QIE_TRY(lm_vector(m, &L.hc_out[q], ph + "out", n));
+            LM_GET(tm, ph + "mix", n, n);
+            QIE_TRY(lm_floats(m, &L.hc_mix[q], *tm));
+        }
+    }
+    if (m->a.canon_taps > 0) {
+        LM_GET(tc, pl + "canon1", (int64_t)m->a.width, (int64_t)m->a.canon_taps);
+        QIE_TRY(lm_floats(m, &L.canon, *tc));
+    }
     if (m->a.block == QIE_BLOCK_SANDWICH) {
         const int64_t Wn = m->a.width;
         QIE_TRY(lm_vector(m, &L.n1, pl + "norm1", Wn));
@@ -417,26 +540,54 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
         QIE_TRY(finalize_mingru(m, i));
         return finalize_ff(m, i);
     }
+    if (d.mixer == QIE_MIXER_CHANNEL_DELTA) {
+        QIE_TRY(finalize_delta(m, i));
+        return finalize_ff(m, i);
+    }
     if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
         QIE_TRY(finalize_gqa_mixer(e, m, i));
         return finalize_ff(m, i);
     }
     const int64_t W = m->a.width, H = d.heads, hq = d.dim + d.rot_dim, R = d.kv_rank;
     const bool own = d.kv_from < 0;
-    LM_GET(tq, px + "q", H * hq, W);
-    LM_GET(tg, px + "g", H, W);
-    const int64_t n_kv = own ? R + d.rot_dim : 0;
-    L.n_in = (int)(H * hq + n_kv + H);
-    L.g_col = (int)(H * hq + n_kv);
-    QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
-    QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tq));
-    if (own) {
-        LM_GET(tk, px + "dkv", R + d.rot_dim, W);
-        LM_GET(tn, px + "dkv.norm", R);
-        QIE_TRY(lm_upload_rows(m, L.w_in, H * hq, W, *tk));
-        QIE_TRY(lm_floats(m, &L.dkv_norm, *tn));
+    const int64_t n_kv = own ? R + d.rot_dim : 0, n_g = d.head_gate ? H : 0;
+    if (d.q_rank > 0) {
+        // first stage [dq ; (dkv)] -> the latent's norm -> W_uq fills the q heads of the projection row
+        QIE_REQUIRE(!d.head_gate, "layer %d: latent queries and the head gate are not wired together", i);
+        const int64_t Q = d.q_rank;
+        L.n_pre = (int)(Q + n_kv);
+        L.n_in = (int)(H * hq);
+        L.g_col = -1;
+        QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_pre * W * m->esz()));
+        LM_GET(tdq, px + "dq", Q, W);
+        QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tdq));
+        QIE_TRY(lm_vector(m, &L.dq_norm, px + "dq.norm", Q));
+        LM_GET(tuq, px + "uq", H * hq, Q);
+        QIE_TRY(lm_alloc(m, &L.w_uq, (size_t)tuq->numel() * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_uq, 0, Q, *tuq));
+        if (own) {
+            LM_GET(tk, px + "dkv", R + d.rot_dim, W);
+            LM_GET(tn, px + "dkv.norm", R);
+            QIE_TRY(lm_upload_rows(m, L.w_in, Q, W, *tk));
+            QIE_TRY(lm_floats(m, &L.dkv_norm, *tn));
+        }
+    } else {
+        LM_GET(tq, px + "q", H * hq, W);
+        L.n_in = (int)(H * hq + n_kv + n_g);
+        L.g_col = n_g ? (int)(H * hq + n_kv) : -1;
+        QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tq));
+        if (own) {
+            LM_GET(tk, px + "dkv", R + d.rot_dim, W);
+            LM_GET(tn, px + "dkv.norm", R);
+            QIE_TRY(lm_upload_rows(m, L.w_in, H * hq, W, *tk));
+            QIE_TRY(lm_floats(m, &L.dkv_norm, *tn));
+        }
+        if (n_g) {
+            LM_GET(tg, px + "g", H, W);
+            QIE_TRY(lm_upload_rows(m, L.w_in, L.g_col, W, *tg));
+        }
     }
-    QIE_TRY(lm_upload_rows(m, L.w_in, L.g_col, W, *tg));
     LM_GET(tuk, px + "uk", H * d.dim, R);
     {   // [heads][dim][R] -> [heads][R][dim]: the absorbed query is q_nope W_uk,h, a product over dim
         std::vector<int64_t> perm((size_t)H * d.dim * R);
@@ -452,7 +603,7 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
     LM_GET(to, px + "o", W, H * d.vdim);
     QIE_TRY(lm_alloc(m, &L.wo, (size_t)to->numel() * m->esz()));
     QIE_TRY(lm_upload_rows(m, L.wo, 0, H * d.vdim, *to));
-    QIE_TRY(lm_rope(m, e, (double)d.rot_base, d.rot_dims, &L.rope));
+    QIE_TRY(lm_rope(m, e, (double)d.rot_base, d.rot_dims, &L.rope, &d.rot_scaling));
     if (m->a.block == QIE_BLOCK_POSTNORM_GAIN) {
         LM_GET(n1, pl + "norm1");
         L.g1 = host_elem(*n1, 0);
@@ -593,6 +744,11 @@ static int enq_latent_post(qie_batch* b, int i, int T) {
     p.cache = cache_of(b);
     p.layer_off = s->layer_off[L.cache_layer];   // engines with latent layers run every layer once: run == layer
     p.interleaved = s->interleaved;
+    p.rot_layout = d.rot_layout;
+    if (d.q_rank > 0 && p.own_kv) {   // the first-stage product holds [latent queries | compressed row | shared key part]
+        p.kv = s->pre + d.q_rank;
+        p.kv_ld = L.n_pre;
+    }
     return lay::latent_post(p, m->f32, T, e->stream);
 }
 
@@ -619,7 +775,8 @@ static int enq_attention(qie_batch* b, int i, int T) {
     p.ld = L.n_in;
     p.row_slot = s->row_slot;
     p.row_pos = s->row_pos;
-    p.heads = d.heads; p.dim = d.dim; p.rot = d.rot_dim; p.R = d.kv_rank; p.window = d.window;
+    const int window = d.window > 0 ? d.window : b->max_ctx;   // 0: every earlier position
+    p.heads = d.heads; p.dim = d.dim; p.rot = d.rot_dim; p.R = d.kv_rank; p.window = window;
     p.scale = d.scale;
     p.cache = cache_of(b);
     p.layer_off = s->layer_off[L.cache_layer];
@@ -630,7 +787,7 @@ static int enq_attention(qie_batch* b, int i, int T) {
         // step has few rows (decoding)
         const int ng = it->second.first;
         int S = 1024 * lay::kLatentQG / ng;
-        const int nb = d.window / 32 + 2;
+        const int nb = window / 32 + 2;
         S = std::max(1, std::min({S, nb, 64}));
         if ((int64_t)ng * S > s->part_cap) {
             hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -652,7 +809,7 @@ static int enq_attention(qie_batch* b, int i, int T) {
         q.row_slot = s->row_slot; q.row_pos = s->row_pos;
         q.groups = s->d_groups + it->second.second;
         q.n_groups = ng; q.S = S;
-        q.heads = d.heads; q.dim = d.dim; q.rot = d.rot_dim; q.R = d.kv_rank; q.window = d.window;
+        q.heads = d.heads; q.dim = d.dim; q.rot = d.rot_dim; q.R = d.kv_rank; q.window = window;
         q.scale = d.scale;
         q.cache = p.cache; q.layer_off = p.layer_off;
         q.part_o = s->part_o; q.part_ml = s->part_ml; q.out = s->olat;
@@ -715,6 +872,7 @@ static int enq_mixer_out(qie_batch* b, int i, int T) {
     const int64_t HR = (int64_t)d.heads * d.kv_rank;
     QIE_TRY(lin(e, s->olat, HR, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank, (int64_t)d.vdim * d.kv_rank,
                 d.vdim));
+    if (L.g_col < 0) return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV);
     QIE_TRY(lay::head_gate(s->ov, s->ov_bf, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
     return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV, s->ov_bf);
 }
@@ -735,7 +893,7 @@ static int enq_ff(qie_batch* b, int i, int T) {
     }
     if (d.ff_kind == QIE_FF_DENSE) {
         QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, 2 * ff, T, 2 * ff, W, s->y_bf));
-        QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, T, ff, st));
+        QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, T, ff, st, d.ff_act == QIE_ACT_GELU_TANH_GATED ? 1 : 0));
         return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff, s->act_bf);
     }
     const int E = d.experts, top = d.top, n = T * top;
@@ -828,7 +986,9 @@ static lay::GqaAttnP gqa_attn_params(qie_batch* b, int r) {
     p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = L.n_cat; p.out_col = 0;
     p.slopes = a.slope_bias ? L.slopes : nullptr;
     p.pb = a.weights == QIE_WEIGHTS_SIGMOID ? L.pb : nullptr;
-    p.gate_col = a.head_gate ? L.col_gate : -1;
+    p.gate_col = (a.head_gate || a.out_gate) ? L.col_gate : -1;
+    p.gate_elem = a.out_gate ? 1 : 0;
+    p.sink = a.sink ? L.sink : nullptr;
     return p;
 }
 
@@ -866,6 +1026,8 @@ static int enq_gqa_post(qie_batch* b, int r, int T) {
     p.v_transposed = s->v_transposed;
     p.q_temp_every = a.q_temp_every;
     p.q_temp_coef = a.q_temp_coef;
+    p.q_bias = a.qk_bias ? L.q_bias : nullptr;
+    p.k_bias = a.qk_bias ? L.k_bias : nullptr;
     return lay::gqa_post(p, m->f32, T, e->stream);
 }
 
@@ -997,37 +1159,149 @@ static int enq_mingru_mixer(qie_batch* b, int r, int T) {
     return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
 }
 
-// Pre-norm blocks: x += mixer(N1(x)); x += ff(N2(x)), plain weight vectors.  The stream lives in
-// plane 1 of the stack; every residual add is fused with the norm that reads its result (the last
-// kernel of a run makes the next run's input unless the streams are kept).
+// Latent attention of layer run r on the branch input s->y -> s->mix (pre-norm blocks).
+static int enq_latent_proj(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    if (L.d.q_rank <= 0) return dense(b, s->y, W, L.w_in, s->proj, L.n_in, T, L.n_in, W, s->y_bf);
+    // [latent queries | compressed row | shared key part] -> the latent's norm in place -> W_uq
+    QIE_TRY(dense(b, s->y, W, L.w_in, s->pre, L.n_pre, T, L.n_pre, W, s->y_bf));
+    QIE_TRY(lay::rms_rows(s->pre, L.n_pre, 0, L.d.q_rank, L.dq_norm, 0.f, m->a.norm_eps, s->pre, L.n_pre, nullptr, T, e->stream));
+    return dense(b, s->pre, L.n_pre, L.w_uq, s->proj, L.n_in, T, L.n_in, L.d.q_rank);
+}
+
+static int enq_latent_mixer(qie_batch* b, int r, int T) {
+    const int i = b->e->lm->runs[r].layer;
+    QIE_TRY(enq_latent_proj(b, i, T));
+    QIE_TRY(enq_latent_post(b, i, T));
+    QIE_TRY(enq_absorb(b, i, T));
+    QIE_TRY(enq_attention(b, i, T));
+    return enq_mixer_out(b, i, T);
+}
+
+// Gated delta rule of layer run r: fused projection [q ; k ; v ; b ; a1 ; g1] and the second-stage
+// products, then (enq_delta_scan) the short convolutions with silu, the gates, the scan and the gated head norm.
+static int enq_delta_proj(qie_batch* b, int r, int T) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    const qie_delta_desc& c = L.d.delta;
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    QIE_TRY(dense(b, s->y, W, L.w_in, s->proj, L.n_in, T, L.n_in, W, s->y_bf));
+    QIE_TRY(dense(b, s->proj + L.col_a1, L.n_in, L.w_a2, s->qabs, (int64_t)c.heads * c.dim, T, c.heads * c.dim, L.rank_a));
+    return dense(b, s->proj + L.col_g1, L.n_in, L.w_g2, s->aux, (int64_t)c.heads * c.vdim, T, c.heads * c.vdim, L.rank_g);
+}
+
+static int enq_delta_scan(qie_batch* b, int r, int T, bool advance) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    const qie_delta_desc& c = L.d.delta;
+    LayeredBatch* s = b->lb;
+    const int C = 2 * c.kv_heads * c.dim + c.heads * c.vdim;
+    lay::CausalConvP cv{};
+    cv.in = s->proj; cv.ld_in = L.n_in; cv.col = 0; cv.C = C; cv.taps = c.conv; cv.w = L.dl_conv;
+    cv.row_slot = s->row_slot; cv.row_pos = s->row_pos; cv.row_k = s->row_k;
+    cv.state = s->state; cv.slot_stride = s->slot_state; cv.state_off = s->conv_off[r];
+    cv.residual = 0; cv.silu = 1;
+    cv.out = s->pre; cv.ld_out = C; cv.out_bf = nullptr;
+    cv.entries = s->d_ent; cv.n_entries = s->n_ent;
+    QIE_TRY(lay::causal_conv(cv, T, e->stream));
+    if (advance) QIE_TRY(lay::causal_conv_state(cv, e->stream));
+    lay::DeltaPrepP pp{s->pre, C, s->proj, L.n_in, L.col_b, s->qabs, L.dl_dt_bias, L.dl_exp_a, c.heads, c.kv_heads, c.dim, c.vdim};
+    QIE_TRY(lay::delta_prep(pp, T, e->stream));
+    lay::DeltaScanP sp{};
+    sp.qkv = s->pre; sp.ld_qkv = C; sp.beta = s->proj + L.col_b; sp.ld_beta = L.n_in; sp.g = s->qabs;
+    sp.entries = s->d_ent; sp.n_entries = s->n_ent;
+    sp.H = c.heads; sp.G = c.kv_heads; sp.dim = c.dim; sp.vdim = c.vdim;
+    sp.state = s->state; sp.slot_stride = s->slot_state; sp.state_off = s->state_off[r];
+    sp.read_state = 1; sp.write_state = advance ? 1 : 0;
+    sp.out = s->olat;
+    QIE_TRY(lay::delta_scan(sp, e->stream));
+    return lay::head_norm_rows(s->olat, nullptr, L.dl_norm, m->a.norm_eps, 1.0f, c.heads, c.vdim, T, s->ov, s->ov_bf, L.n_cat, 0,
+                               e->stream, s->aux);
+}
+
+static int enq_delta_mixer(qie_batch* b, int r, int T) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    QIE_TRY(enq_delta_proj(b, r, T));
+    QIE_TRY(enq_delta_scan(b, r, T, true));
+    return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
+}
+
+// Pre-norm blocks: x += mixer(N1(x)); x += ff(N2(x)) with weights norm_offset + w.  One residual row
+// (streams 0): the stream lives in plane 1 of the stack and every residual add is fused with the norm
+// that reads its result.  Several rows (hyper-connections): planes 0 .. streams - 1; the update after
+// a sublayer, the read-out for the next one and its norm are one kernel.  Either way the last kernel
+// of a run makes the next run's input.  With an input convolution the mixer's normed input goes to
+// s->x first and h + conv(h) to s->y.
 static int enq_run_prenorm(qie_batch* b, int r, int T, bool h_ready, bool* next_ready) {
     const qie_engine* e = b->e;
     const LayeredModel* m = e->lm;
     const LayerDev& L = m->L[m->runs[r].layer];
     LayeredBatch* s = b->lb;
-    const int W = m->a.width;
+    const int W = m->a.width, n = m->a.streams;
     hipStream_t st = e->stream;
-    float* x = s->stack + s->cap * W;
-    const float eps = m->a.norm_eps;
-    if (!h_ready) QIE_TRY(lay::add_norm(x, x, nullptr, nullptr, nullptr, L.n1, s->y, s->y_bf, T, W, eps, st, 0.f));
-    if (L.d.mixer == QIE_MIXER_MINGRU)
-        QIE_TRY(enq_mingru_mixer(b, r, T));
-    else
-        QIE_TRY(enq_gqa_mixer(b, r, T));
+    const int64_t plane = s->cap * W;
+    float* x = n > 0 ? s->stack : s->stack + plane;
+    const float eps = m->a.norm_eps, w_one = m->a.norm_offset;
+    const bool canon = m->a.canon_taps > 0;
+    // y: the sublayer result that updates the rows with the coefficients of sublayer q of this layer (null:
+    // none); then the read-out with in_next (hyper-connections) normed with wn -> h (null wn: no read-out)
+    auto step = [&](const float* y, int q, const float* in_next, const float* wn, bool to_mixer, float* sum) -> int {
+        float* h = to_mixer && canon ? s->x : s->y;
+        uint16_t* h_bf = to_mixer && canon ? nullptr : s->y_bf;
+        if (n > 0) {
+            lay::StreamStepP p{x, plane, n, y, y ? L.hc_mix[q] : nullptr, y ? L.hc_out[q] : nullptr, wn ? in_next : nullptr, wn, w_one, eps,
+                               h, h_bf, sum, T, W};
+            return lay::stream_step(p, st);
+        }
+        return lay::add_norm(x, x, y, nullptr, nullptr, wn, h, h_bf, T, W, eps, st, w_one);
+    };
+    if (!h_ready) QIE_TRY(step(nullptr, 0, L.hc_in[0], L.n1, true, nullptr));
+    if (canon) {
+        lay::CausalConvP cv{};
+        cv.in = s->x; cv.ld_in = W; cv.col = 0; cv.C = W; cv.taps = m->a.canon_taps; cv.w = L.canon;
+        cv.row_slot = s->row_slot; cv.row_pos = s->row_pos; cv.row_k = s->row_k;
+        cv.state = s->state; cv.slot_stride = s->slot_state; cv.state_off = s->canon_off[r];
+        cv.residual = 1; cv.silu = 0;
+        cv.out = s->y; cv.ld_out = W; cv.out_bf = s->y_bf;
+        cv.entries = s->d_ent; cv.n_entries = s->n_ent;
+        QIE_TRY(lay::causal_conv(cv, T, st));
+        QIE_TRY(lay::causal_conv_state(cv, st));
+    }
+    switch (L.d.mixer) {
+        case QIE_MIXER_MINGRU: QIE_TRY(enq_mingru_mixer(b, r, T)); break;
+        case QIE_MIXER_LATENT_ATTENTION: QIE_TRY(enq_latent_mixer(b, r, T)); break;
+        case QIE_MIXER_CHANNEL_DELTA: QIE_TRY(enq_delta_mixer(b, r, T)); break;
+        default: QIE_TRY(enq_gqa_mixer(b, r, T)); break;
+    }
     const bool has_ff = L.d.ff_kind != QIE_FF_NONE;
     const bool last = r + 1 == (int)m->runs.size();
-    const bool fuse_next = !last && !s->keep_on;
-    const float* next_w = fuse_next ? m->L[m->runs[r + 1].layer].n1 : nullptr;
+    // several rows: the kept stream of a run is the rows' sum, an extra output of the run's last kernel
+    const bool fuse_next = !last && (n > 0 || !s->keep_on);
+    const LayerDev* N = last ? nullptr : &m->L[m->runs[r + 1].layer];
+    const float* next_w = fuse_next ? N->n1 : nullptr;
+    const float* next_in = fuse_next ? N->hc_in[0] : nullptr;
+    float* sum = n > 0 ? (s->keep_on && s->keep ? s->keep + (int64_t)r * plane : last ? s->x : nullptr) : nullptr;
     if (has_ff) {
-        QIE_TRY(lay::add_norm(x, x, s->mix, nullptr, nullptr, L.n2, s->y, s->y_bf, T, W, eps, st, 0.f));
+        QIE_TRY(step(s->mix, 0, L.hc_in[1], L.n2, false, nullptr));
         QIE_TRY(enq_ff(b, m->runs[r].layer, T));
-        QIE_TRY(lay::add_norm(x, x, s->ffo, nullptr, nullptr, next_w, s->y, s->y_bf, T, W, eps, st, 0.f));
+        QIE_TRY(step(s->ffo, 1, next_in, next_w, true, sum));
     } else {
-        QIE_TRY(lay::add_norm(x, x, s->mix, nullptr, nullptr, next_w, s->y, s->y_bf, T, W, eps, st, 0.f));
+        QIE_TRY(step(s->mix, 0, next_in, next_w, true, sum));
     }
     *next_ready = fuse_next;
-    if (s->keep_on && s->keep)
-        QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)r * s->cap * W, x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    if (n > 0) {
+        if (last && sum != s->x) QIE_HIP(hipMemcpyAsync(s->x, sum, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    } else if (s->keep_on && s->keep) {
+        QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)r * plane, x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    }
     return 0;
 }
 
@@ -1106,14 +1380,22 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     LayeredBatch* s = b->lb;
     const int W = m->a.width;
     const float* x = s->stack;
-    const float w_one = m->a.block == QIE_BLOCK_PRENORM ? 0.f : 1.f;
+    const float w_one = m->a.block == QIE_BLOCK_PRENORM ? m->a.norm_offset : 1.f;
     if (m->a.block == QIE_BLOCK_PRENORM) {
-        float* xs = s->stack + s->cap * W;
-        QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, xs, nullptr, T, W, m->a.vocab, e->stream, m->a.embed_scale,
+        // one residual row: plane 1; several: planes 0 .. streams - 1, all equal to the embedding output
+        const int n = m->a.streams;
+        const int64_t plane = s->cap * W;
+        float* xs = n > 0 ? s->stack : s->stack + plane;
+        float* raw = m->a.embed_norm ? s->mix : xs;
+        QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, raw, nullptr, T, W, m->a.vocab, e->stream, m->a.embed_scale,
                                 m->a.pos_embed == QIE_POS_SINUSOID ? s->row_pos : nullptr, m->pos_freq));
+        if (m->a.embed_norm)
+            QIE_TRY(lay::add_norm(raw, raw, nullptr, nullptr, nullptr, m->w_embed, xs, nullptr, T, W, m->a.norm_eps, e->stream,
+                                  m->a.norm_offset));
+        for (int k = 1; k < n; k++) QIE_HIP(hipMemcpyAsync(xs + k * plane, xs, (size_t)T * W * 4, hipMemcpyDeviceToDevice, e->stream));
         bool ready = false;
         for (int r = 0; r < (int)m->runs.size(); r++) QIE_TRY(enq_run_prenorm(b, r, T, ready, &ready));
-        x = xs;
+        x = n > 0 ? s->x : xs;
     } else if (m->a.block == QIE_BLOCK_SANDWICH) {
         // the embedding rows stay in plane 0 only when a repeated group adds them again
         float* xs = s->stack + s->cap * W;
@@ -1146,13 +1428,14 @@ static void lb_free(LayeredBatch* s) {
     drop_graphs(s);   // captured launches hold these buffers' addresses
     void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
                   s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf,
-                  s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf};
+                  s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf, s->pre, s->aux, s->row_k};
     for (void* p : ps)
         if (p) hipFree(p);
     s->stack = s->x = s->proj = s->qabs = s->olat = s->ov = s->mix = s->y = s->gu = s->act = s->ffo = s->xg = s->yd = s->score =
         s->keep = nullptr;
     s->abf = s->x_bf = s->y_bf = s->ov_bf = s->act_bf = s->xg_bf = nullptr;
-    s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = nullptr;
+    s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = s->row_k = nullptr;
+    s->pre = s->aux = nullptr;
     s->cap = 0;
 }
 
@@ -1215,11 +1498,14 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         auto A = [&](void** p, int64_t elems, size_t sz = 4) {
             if (!rc) rc = dmalloc(p, (size_t)elems * sz);
         };
-        A((void**)&s->stack, (m->a.depth_mix ? L + 1 : 2) * cap * W);
+        A((void**)&s->stack, (m->a.depth_mix ? L + 1 : std::max<int64_t>(2, m->a.streams)) * cap * W);
+        A((void**)&s->pre, cap * std::max<int64_t>(s->m_pre, 1));
+        A((void**)&s->aux, cap * std::max<int64_t>(s->m_aux, 1));
+        A((void**)&s->row_k, cap);
         A((void**)&s->x, cap * W);
         A((void**)&s->proj, cap * s->m_in);
-        A((void**)&s->qabs, cap * s->m_hr);
-        A((void**)&s->olat, cap * s->m_hr);
+        A((void**)&s->qabs, cap * std::max<int64_t>(s->m_hr, 1));
+        A((void**)&s->olat, cap * std::max<int64_t>(s->m_hr, 1));
         A((void**)&s->ov, cap * s->m_hv);
         A((void**)&s->mix, cap * W);
         A((void**)&s->y, cap * W);
@@ -1254,7 +1540,7 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         if (s->h_stage) hipHostFree(s->h_stage);
         s->h_stage = nullptr;
         const int64_t rows = (T + 255) / 256 * 256;
-        QIE_HIP(hipHostMalloc((void**)&s->h_stage, (size_t)rows * 3 * 4, hipHostMallocDefault));
+        QIE_HIP(hipHostMalloc((void**)&s->h_stage, (size_t)rows * 4 * 4, hipHostMallocDefault));
         s->h_stage_rows = rows;
     }
     return 0;
@@ -1309,6 +1595,8 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     s->layer_off.assign(n_runs, 0);
     s->v_off.assign(n_runs, 0);
     s->state_off.assign(n_runs, 0);
+    s->conv_off.assign(n_runs, 0);
+    s->canon_off.assign(n_runs, 0);
     // bf16 caches whose every layer fits the matrix-core attention carry, after the rows of a
     // caching layer, the key-interleaved copy of c (R more elements per token)
     s->interleaved = !m->f32;
@@ -1320,7 +1608,7 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     s->v_transposed = !m->f32;
     for (int i = 0; i < m->a.n_layers; i++) {
         const qie_layer_desc& d = m->L[i].d;
-        if (d.mixer == QIE_MIXER_MINGRU) continue;   // caches nothing
+        if (d.mixer == QIE_MIXER_MINGRU || d.mixer == QIE_MIXER_CHANNEL_DELTA) continue;   // cache nothing
         if (d.mixer == QIE_MIXER_LATENT_ATTENTION || !lay::gqa_attention_mfma_fits(d.gqa.dim, d.gqa.vdim, page_tokens))
             s->v_transposed = false;
         if (d.mixer != QIE_MIXER_LATENT_ATTENTION) s->m_vd = std::max<int64_t>(s->m_vd, d.gqa.vdim);
@@ -1329,7 +1617,25 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     for (int r = 0; r < n_runs; r++) {
         const int i = m->runs[r].layer;
         const qie_layer_desc& d = m->L[i].d;
-        if (d.mixer == QIE_MIXER_MINGRU) {
+        if (m->a.canon_taps > 1) {   // the last taps - 1 normed mixer inputs of every run
+            s->canon_off[r] = s->slot_state;
+            s->slot_state += (int64_t)(m->a.canon_taps - 1) * m->a.width;
+        }
+        if (d.mixer == QIE_MIXER_CHANNEL_DELTA) {
+            // no cache rows; per slot the heads' states and the short convolutions' last inputs
+            const qie_delta_desc& c = d.delta;
+            const int64_t C = 2 * (int64_t)c.kv_heads * c.dim + (int64_t)c.heads * c.vdim;
+            s->state_off[r] = s->slot_state;
+            s->slot_state += (int64_t)c.heads * c.dim * c.vdim;
+            s->conv_off[r] = s->slot_state;
+            s->slot_state += (int64_t)(c.conv - 1) * C;
+            s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
+            s->m_pre = std::max<int64_t>(s->m_pre, C);
+            s->m_hr = std::max<int64_t>({s->m_hr, (int64_t)c.heads * c.dim, (int64_t)c.heads * c.vdim});
+            s->m_aux = std::max<int64_t>(s->m_aux, (int64_t)c.heads * c.vdim);
+            s->m_hv = std::max<int64_t>(s->m_hv, (int64_t)c.heads * c.vdim);
+            s->m_abf = std::max<int64_t>({s->m_abf, (int64_t)m->a.width, (int64_t)c.heads * c.vdim});
+        } else if (d.mixer == QIE_MIXER_MINGRU) {
             // no cache rows; `width` state elements per slot
             const int64_t n = d.mingru.width;
             s->state_off[r] = s->slot_state;
@@ -1380,6 +1686,8 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
         }
         const int64_t H = d.heads;
         s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
+        s->m_pre = std::max<int64_t>(s->m_pre, m->L[i].n_pre);
+        s->m_abf = std::max<int64_t>(s->m_abf, d.q_rank);
         s->m_hr = std::max<int64_t>(s->m_hr, H * d.kv_rank);
         s->m_r = std::max<int64_t>(s->m_r, d.kv_rank);
         s->m_hv = std::max<int64_t>(s->m_hv, H * d.vdim);
@@ -1473,6 +1781,12 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
                 "qie_engine_create_layered: repeated group [%d, %d) x %d of %d layers", arch->loop_start, arch->loop_stop,
                 arch->loop_times, arch->n_layers);
     QIE_REQUIRE(!loops || arch->block == QIE_BLOCK_SANDWICH, "qie_engine_create_layered: repeated groups go with the sandwich block");
+    QIE_REQUIRE(arch->streams >= 0 && arch->streams <= 8 && arch->canon_taps >= 0 && arch->canon_taps <= 64,
+                "qie_engine_create_layered: %d residual streams (at most 8), %d input taps (at most 64)", arch->streams, arch->canon_taps);
+    QIE_REQUIRE(arch->block == QIE_BLOCK_PRENORM || (arch->streams == 0 && arch->canon_taps == 0 && !arch->embed_norm &&
+                                                     arch->norm_offset == 0.f),
+                "qie_engine_create_layered: residual streams, the input convolution, the embedding norm and the norm offset "
+                "go with the pre-norm block");
     for (int i = 0; i < arch->n_layers; i++) {
         const qie_layer_desc& d = arch->layers[i];
         QIE_REQUIRE(d.ff_kind >= QIE_FF_NONE && d.ff_kind <= QIE_FF_MOE, "layer %d: unknown feed-forward %d", i, d.ff_kind);
@@ -1480,7 +1794,7 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
         QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts + std::max(d.identity, 0)),
                     "layer %d: %d of %d experts", i, d.top, d.experts + std::max(d.identity, 0));
         QIE_REQUIRE(d.router >= QIE_ROUTER_SIGMOID_IN && d.router <= QIE_ROUTER_SOFTMAX_ALL, "layer %d: router %d", i, d.router);
-        QIE_REQUIRE(d.ff_act == QIE_ACT_SILU_GATED || d.ff_act == QIE_ACT_XIELU, "layer %d: activation %d", i, d.ff_act);
+        QIE_REQUIRE(d.ff_act >= QIE_ACT_SILU_GATED && d.ff_act <= QIE_ACT_GELU_TANH_GATED, "layer %d: activation %d", i, d.ff_act);
         if (d.ff_kind == QIE_FF_MOE && d.router == QIE_ROUTER_SOFTMAX_ALL) {
             const int n = d.experts + d.identity;
             QIE_REQUIRE(d.identity >= 0 && d.groups >= 1 && n % d.groups == 0 && d.groups_keep >= 1 && d.groups_keep <= d.groups &&
@@ -1493,6 +1807,15 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
         if (d.mixer == QIE_MIXER_MINGRU) {
             QIE_REQUIRE(arch->block == QIE_BLOCK_PRENORM, "layer %d: this mixer is wired to the pre-norm block", i);
             QIE_REQUIRE(d.mingru.width > 0, "layer %d: minGRU width", i);
+            continue;
+        }
+        if (d.mixer == QIE_MIXER_CHANNEL_DELTA) {
+            const qie_delta_desc& c = d.delta;
+            QIE_REQUIRE(arch->block == QIE_BLOCK_PRENORM, "layer %d: this mixer is wired to the pre-norm block", i);
+            QIE_REQUIRE(c.heads > 0 && c.kv_heads > 0 && c.heads % c.kv_heads == 0 && c.dim > 0 && c.dim <= 512 && c.vdim > 0 &&
+                            c.conv >= 1 && c.conv <= 64 && c.rank_a >= 0 && c.rank_g >= 0,
+                        "layer %d: delta rule with %d heads over %d key heads of %d (at most 512) / %d, %d taps", i, c.heads, c.kv_heads,
+                        c.dim, c.vdim, c.conv);
             continue;
         }
         if (d.mixer == QIE_MIXER_GQA || d.mixer == QIE_MIXER_GQA_RECURRENT) {
@@ -1514,22 +1837,31 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
             QIE_REQUIRE(a.mask >= QIE_MASK_CAUSAL && a.mask <= QIE_MASK_CHUNK && (a.mask == QIE_MASK_CAUSAL || a.mask_size > 0),
                         "layer %d: mask %d of size %d", i, a.mask, a.mask_size);
             QIE_REQUIRE(!a.values_are_keys || (a.vdim == a.dim && !a.rot_values), "layer %d: keys as values need vdim == dim", i);
+            QIE_REQUIRE(!(a.out_gate && a.head_gate), "layer %d: one output gate, per head or per coordinate", i);
+            QIE_REQUIRE(!a.sink || a.weights == QIE_WEIGHTS_SOFTMAX, "layer %d: a sink goes with softmax weights", i);
+            QIE_REQUIRE(a.rot_scaling.factor == 0.f || (a.rot_scaling.factor > 0.f && a.rot_scaling.high > a.rot_scaling.low &&
+                                                        a.rot_scaling.low >= 0.f && a.rot_scaling.original > 0.f),
+                        "layer %d: rotary scaling", i);
             if (d.mixer == QIE_MIXER_GQA_RECURRENT)
                 QIE_REQUIRE(d.rec.heads > 0 && d.rec.dim > 0 && d.rec.dim <= 512 && d.rec.vdim > 0, "layer %d: recurrence sizes", i);
             continue;
         }
         QIE_REQUIRE(d.mixer == QIE_MIXER_LATENT_ATTENTION, "layer %d: unknown mixer %d", i, d.mixer);
-        QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN, "layer %d: latent attention is wired to the post-norm block", i);
-        QIE_REQUIRE(d.heads > 0 && d.dim > 0 && d.rot_dim >= 0 && d.vdim > 0 && d.kv_rank > 0 && d.window > 0,
+        QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN || arch->block == QIE_BLOCK_PRENORM,
+                    "layer %d: latent attention is wired to the post-norm and pre-norm blocks", i);
+        QIE_REQUIRE(d.heads > 0 && d.dim > 0 && d.rot_dim >= 0 && d.vdim > 0 && d.kv_rank > 0 && d.window >= 0 && d.q_rank >= 0,
                     "layer %d: invalid mixer sizes", i);
+        QIE_REQUIRE(d.rot_layout == QIE_ROT_HALVES || d.rot_layout == QIE_ROT_INTERLEAVED, "layer %d: rotary layout %d", i, d.rot_layout);
+        QIE_REQUIRE(d.q_rank == 0 || !d.head_gate, "layer %d: latent queries and the head gate are not wired together", i);
         QIE_REQUIRE(d.rot_dims >= 0 && d.rot_dims % 2 == 0 && d.rot_dims <= d.rot_dim, "layer %d: rotary dims %d of %d", i,
                     d.rot_dims, d.rot_dim);
         QIE_REQUIRE(d.rot_dims == 0 || d.rot_base > 0.f, "layer %d: rotary base", i);
         if (d.kv_from >= 0) {
             QIE_REQUIRE(d.kv_from < i, "layer %d: kv_from %d must name an earlier layer", i, d.kv_from);
             const qie_layer_desc& o = arch->layers[d.kv_from];
-            QIE_REQUIRE(o.kv_from < 0 && o.kv_rank == d.kv_rank && o.rot_dim == d.rot_dim && o.rot_dims == d.rot_dims &&
-                            o.rot_base == d.rot_base,
+            QIE_REQUIRE(o.mixer == QIE_MIXER_LATENT_ATTENTION && o.kv_from < 0 && o.kv_rank == d.kv_rank && o.rot_dim == d.rot_dim &&
+                            o.rot_dims == d.rot_dims && o.rot_base == d.rot_base && o.rot_layout == d.rot_layout &&
+                            memcmp(&o.rot_scaling, &d.rot_scaling, sizeof(qie_rot_scaling)) == 0,
                         "layer %d: the layer it reads its cache from (%d) must own one of the same shape and rotation", i,
                         d.kv_from);
         }
@@ -1614,6 +1946,7 @@ int qie_engine_finalize_weights(qie_engine* e) {
         QIE_TRY(lm_alloc(m, (void**)&m->pos_freq, fr.size() * 8));
         QIE_HIP(hipMemcpy(m->pos_freq, fr.data(), fr.size() * 8, hipMemcpyHostToDevice));
     }
+    if (m->a.embed_norm) QIE_TRY(lm_vector(m, &m->w_embed, "embed.norm", W));
     if (m->a.block == QIE_BLOCK_SANDWICH || m->a.block == QIE_BLOCK_PRENORM) {
         QIE_TRY(lm_vector(m, &m->w_final, "final.norm", W));
     } else {
@@ -1669,6 +2002,7 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
             hs[r] = sl;
             hs[R + r] = b->h_pos[sl] + k;
             hs[2 * R + r] = tokens[r];
+            hs[3 * R + r] = k;
         }
         b->h_pos[sl] += counts[i];
     }
@@ -1737,6 +2071,7 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
     QIE_HIP(hipMemcpyAsync(s->row_slot, hs, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->row_pos, hs + R, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->tok, hs + 2 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
+    QIE_HIP(hipMemcpyAsync(s->row_k, hs + 3 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_TRY(build_groups(b, n_entries, counts));
     if (n_want > 0) QIE_HIP(hipMemcpyAsync(s->want, want_rows, (size_t)n_want * 4, hipMemcpyHostToDevice, st));
     QIE_TRY(run_forward(b, (int)T, n_want));
@@ -1816,13 +2151,35 @@ int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t ite
     QIE_HIP(hipEventCreate(&e1));
     int rc = 0;
     const bool gqa = which != 0 && m->L[layer].d.mixer != QIE_MIXER_LATENT_ATTENTION;
-    QIE_REQUIRE(which != 4 || m->L[layer].d.mixer == QIE_MIXER_GQA_RECURRENT || m->L[layer].d.mixer == QIE_MIXER_MINGRU,
+    QIE_REQUIRE(which != 4 || m->L[layer].d.mixer == QIE_MIXER_GQA_RECURRENT || m->L[layer].d.mixer == QIE_MIXER_MINGRU ||
+                    m->L[layer].d.mixer == QIE_MIXER_CHANNEL_DELTA,
                 "qie_batch_time_stage: layer %d has no recurrence", layer);
-    QIE_REQUIRE(which != 1 || m->L[layer].d.mixer != QIE_MIXER_MINGRU, "qie_batch_time_stage: layer %d has no attention", layer);
+    QIE_REQUIRE(which != 1 || (m->L[layer].d.mixer != QIE_MIXER_MINGRU && m->L[layer].d.mixer != QIE_MIXER_CHANNEL_DELTA),
+                "qie_batch_time_stage: layer %d has no attention", layer);
     int run = 0;   // the layer's first run
     while (which != 0 && m->runs[run].layer != layer) run++;
     auto once = [&]() -> int {
         const float* xin = layer == 0 || which == 0 ? s->stack : s->x;
+        if (gqa && m->L[layer].d.mixer == QIE_MIXER_CHANNEL_DELTA) {   // the slots' states are read, not advanced
+            const LayerDev& L = m->L[layer];
+            switch (which) {
+                case 2:
+                    QIE_TRY(enq_delta_proj(b, run, T));
+                    return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
+                case 3: return enq_ff(b, layer, T);
+                default: return enq_delta_scan(b, run, T, false);
+            }
+        }
+        if (!gqa && which != 0 && m->a.block == QIE_BLOCK_PRENORM) {   // latent attention on the branch input s->y
+            switch (which) {
+                case 1: return enq_attention(b, layer, T);
+                case 2:
+                    QIE_TRY(enq_latent_proj(b, layer, T));
+                    QIE_TRY(enq_absorb(b, layer, T));
+                    return enq_mixer_out(b, layer, T);
+                default: return enq_ff(b, layer, T);
+            }
+        }
         if (gqa) {   // the recurrence is timed from a zero state over the step's rows, the slots' states are not kept
             const LayerDev& L = m->L[layer];
             switch (which) {

@@ -334,16 +334,17 @@ __global__ __launch_bounds__(256) void latent_post_kernel(LatentPostP p) {
     const float* cs = p.rope_cos + (int64_t)pos * half;
     const float* sn = p.rope_sin + (int64_t)pos * half;
     const int hq = p.dim + p.rot;
-    // queries: rotate the rotated part of every head in place
+    // queries: rotate the rotated part of every head in place; pair j is (j, j + half) or (2j, 2j + 1)
+    const int ia = p.rot_layout ? 2 : 1, ib = p.rot_layout ? 1 : half;
     for (int i = tid; i < p.heads * half; i += 256) {
         const int h = i / half, j = i % half;
         float* q = row + h * hq + p.dim;
-        const float u = q[j], v = q[j + half];
-        q[j] = u * cs[j] - v * sn[j];
-        q[j + half] = v * cs[j] + u * sn[j];
+        const float u = q[j * ia], v = q[j * ia + ib];
+        q[j * ia] = u * cs[j] - v * sn[j];
+        q[j * ia + ib] = v * cs[j] + u * sn[j];
     }
     if (!p.own_kv) return;
-    const float* d = row + p.heads * hq;
+    const float* d = p.kv ? p.kv + (int64_t)t * p.kv_ld : row + p.heads * hq;
     float ss = 0.f;
     for (int i = tid; i < p.R; i += 256) ss += d[i] * d[i];
     ss = block_sum256(ss, red);
@@ -361,12 +362,14 @@ __global__ __launch_bounds__(256) void latent_post_kernel(LatentPostP p) {
     const float* kr = d + p.R;
     for (int j = tid; j < p.rot; j += 256) {
         float v;
-        if (j < half)
-            v = kr[j] * cs[j] - kr[j + half] * sn[j];
-        else if (j < p.rot_dims)
-            v = kr[j] * cs[j - half] + kr[j - half] * sn[j - half];
-        else
+        if (j >= p.rot_dims)
             v = kr[j];
+        else if (p.rot_layout)
+            v = (j & 1) ? kr[j] * cs[j >> 1] + kr[j - 1] * sn[j >> 1] : kr[j] * cs[j >> 1] - kr[j + 1] * sn[j >> 1];
+        else if (j < half)
+            v = kr[j] * cs[j] - kr[j + half] * sn[j];
+        else
+            v = kr[j] * cs[j - half] + kr[j - half] * sn[j - half];
         stf<TC>(out, p.R + j, v);
     }
 }
@@ -556,20 +559,21 @@ int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* 
 
 // ------------------------------------------------------------------ gated activation
 // a[m, j] = silu(gu[m, j]) * gu[m, ff + j]
-__global__ __launch_bounds__(256) void silu_mul_kernel(const float* gu, float* a, uint16_t* a_bf, int ff, int64_t n) {
+// (act 1: the tanh form of gelu instead of silu, gelu(g) = g / 2 (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))))
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* gu, float* a, uint16_t* a_bf, int ff, int64_t n, int act) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const int64_t m = i / ff;
     const int j = (int)(i % ff);
     const float g = gu[m * 2 * ff + j], u = gu[m * 2 * ff + ff + j];
-    const float o = g / (1.0f + expf(-g)) * u;
+    const float o = (act == 1 ? 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) : g / (1.0f + expf(-g))) * u;
     a[i] = o;
     if (a_bf) a_bf[i] = f2bf(o);
 }
-int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st) {
+int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st, int act) {
     const int64_t n = M * ff;
     if (n == 0) return 0;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, a_bf, ff, n);
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, a_bf, ff, n, act);
     QIE_LAUNCH_CHECK();
     return 0;
 }

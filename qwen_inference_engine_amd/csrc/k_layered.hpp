@@ -51,6 +51,9 @@ struct LatentPostP {
     LatentCache cache;
     int64_t layer_off;
     int interleaved;      // bf16 caches: also write the key-interleaved copy of c that follows the rows
+    int rot_layout;       // 0: coordinate i turns with i + rot_dims / 2; 1: 2i with 2i + 1
+    const float* kv;      // own_kv: where the compressed row and the shared key part are read from
+    int64_t kv_ld;        //   ([T][kv_ld], columns 0 .. R + rot); null: the projection row after the q heads
 };
 int latent_post(const LatentPostP& p, bool cache_f32, int T, hipStream_t st);
 
@@ -130,6 +133,8 @@ struct GqaPostP {
     // the division rounded down
     int q_temp_every;
     float q_temp_coef;
+    const float* q_bias;      // [heads * dim] / [kv_heads * dim] or null: added to q / k as they leave the projection
+    const float* k_bias;      //   (a key cached as the value carries its bias)
 };
 int gqa_post(const GqaPostP& p, bool cache_f32, int T, hipStream_t st);
 
@@ -164,6 +169,8 @@ struct GqaAttnP {
     const float* pb;          // [heads] or null; set: a visible key's weight is sigmoid(score + pb[h]),
                               // and the weights of a row are used as they are (no softmax)
     int gate_col;             // >= 0: head h's result times sigmoid(proj[t * ld + gate_col + h])
+    int gate_elem;            // with gate_col: one gate per coordinate, proj[t * ld + gate_col + h * vdim + c]
+    const float* sink;        // [heads] or null: exp(sink[h]) joins the softmax denominator (no key, no value)
 };
 int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);
 // The matrix-core form for bf16 caches whose V rows are stored transposed (v_transposed: inside a
@@ -276,8 +283,97 @@ struct MinGruCarryP {
 };
 int mingru_carry(const MinGruCarryP& p, hipStream_t st);
 
+// gate (optional, [T][heads * vdim]): the result is also multiplied by sigmoid(gate[t, h * vdim + c])
 int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
-                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st);
+                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st, const float* gate = nullptr);
+
+// ------------------------------------------------------------------ residual streams (k_streams.hip)
+// n residual rows per token, X + s * plane (rows of W).  With y (a sublayer's result, [T][W]) the rows
+// are replaced, all at once from the old ones, by x_t = sum_s mix[s * n + t] x_s + out[t] y.  With `in`
+// the read-out u = sum_s in[s] x_s of the (new) rows is normed, h = u / sqrt(mean(u^2) + eps) *
+// (w_one + wn), with its bf16 image.  sum (optional) receives the plain sum of the (new) rows.
+struct StreamStepP {
+    float* X;
+    int64_t plane;
+    int n;
+    const float* y;
+    const float* mix;
+    const float* out;
+    const float* in;
+    const float* wn;
+    float w_one, eps;
+    float* h;
+    uint16_t* h_bf;
+    float* sum;
+    int T, W;
+};
+int stream_step(const StreamStepP& p, hipStream_t st);
+
+// Causal convolution over time per channel on the packed rows of a step: out[t, c] =
+// (residual ? in[t, c] : 0) + sum_j w[c * taps + j] in[t - (taps - 1 - j), c], then silu when asked.
+// Rows before an entry's first come from the slot's state ([taps - 1][C] floats at state + slot *
+// slot_stride + state_off: the inputs at the taps - 1 positions before the entry, oldest first), rows
+// before position 0 are zero.  row_k: a row's index inside its entry.  causal_conv_state moves the
+// state on by the step's entries {first packed row, rows, slot, first position}; run it after
+// causal_conv (which reads the old state) and before `in` is overwritten.
+struct CausalConvP {
+    const float* in;
+    int64_t ld_in;
+    int col, C, taps;
+    const float* w;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    const int32_t* row_k;
+    float* state;
+    int64_t slot_stride, state_off;
+    int residual, silu;
+    float* out;
+    int64_t ld_out;
+    uint16_t* out_bf;
+    const int4* entries;
+    int n_entries;
+};
+int causal_conv(const CausalConvP& p, int T, hipStream_t st);
+int causal_conv_state(const CausalConvP& p, hipStream_t st);
+// out[t, c] = in[t, col + c] / sqrt(mean_c in^2 + eps) * (w_one + w[c]), c < n (out may be in + col)
+int rms_rows(const float* in, int64_t ld_in, int col, int n, const float* w, float w_one, float eps, float* out, int64_t ld_out,
+             uint16_t* out_bf, int T, hipStream_t st);
+
+// ------------------------------------------------------------------ gated delta rule (k_delta.hip)
+// qkv [T][ld_qkv]: q (G heads of dim), k (G x dim), v (H x vdim) after their convolutions.  delta_prep,
+// in place: q and k heads to unit length (x / sqrt(sum x^2 + 1e-6)), q also times dim^(-1/2);
+// proj[t, b_col + h] = sigmoid of itself; a [T][H * dim] = exp(-exp_a[h] * softplus(a + dt_bias)).
+struct DeltaPrepP {
+    float* qkv;
+    int64_t ld_qkv;
+    float* proj;
+    int64_t ld;
+    int b_col;
+    float* a;
+    const float* dt_bias;   // [H * dim]
+    const float* exp_a;     // [H]: exp(A_log)
+    int H, G, dim, vdim;
+};
+int delta_prep(const DeltaPrepP& p, int T, hipStream_t st);
+// Per entry {first packed row, rows, slot, first position} and head h (key head h / (H / G)), the fp32
+// state S [dim][vdim] at state + slot * slot_stride + state_off + h * dim * vdim walks the rows in
+// order: S = diag(g) S; u = beta (v - S^T k); S += k u^T; out[t, h] = S^T q.  An entry whose first
+// position is 0 (or read_state = 0) starts from S = 0; write_state = 0 leaves the slot's state alone.
+struct DeltaScanP {
+    const float* qkv;
+    int64_t ld_qkv;
+    const float* beta;      // beta[t * ld_beta + h]
+    int64_t ld_beta;
+    const float* g;         // [T][H * dim]
+    const int4* entries;
+    int n_entries;
+    int H, G, dim, vdim;
+    float* state;
+    int64_t slot_stride, state_off;
+    int read_state, write_state;
+    float* out;             // [T][H * vdim]
+};
+int delta_scan(const DeltaScanP& p, hipStream_t st);
 // Rows of W: x = xin + (wb ? rms(v) * (w_one + wb) : v) (when v) + add (when add); then (when wn)
 // h = rms(x) * (w_one + wn) with its bf16 image.  xin may be x.  w_one = 1: weight vectors stored
 // around zero; 0: plain weights.
@@ -297,7 +393,8 @@ int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T
 int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, const float* w1p,
                float eps, hipStream_t st, float w_one = 1.0f);
 int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, uint16_t* x_bf, int64_t count, hipStream_t st);
-int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st);
+// a[m, j] = act(gu[m, j]) * gu[m, ff + j]; act 0: silu, 1: the tanh form of gelu
+int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st, int act = 0);
 // a = ap u^2 + u / 2 where u > 0, else aq (exp(u) - 1 - u) + u / 2; n elements
 int xielu(const float* u, float* a, uint16_t* a_bf, int64_t n, float ap, float aq, hipStream_t st);
 // mode 0: score = sigmoid(z) of the `top` largest z = W_r y; mode 1: z = W_r y + bias, score = the

@@ -107,10 +107,11 @@ __global__ __launch_bounds__(256) void gqa_post_kernel(GqaPostP p) {
         const int hh = h0 + wave;
         const bool on = hh < H + G, is_q = hh < H;
         float* x = row + (is_q ? p.q_col + hh * dim : p.k_col + (hh - H) * dim);
+        const float* bias = !on ? nullptr : is_q ? (p.q_bias ? p.q_bias + hh * dim : nullptr) : (p.k_bias ? p.k_bias + (hh - H) * dim : nullptr);
         if (on) {
             float ss = 0.f;
             for (int i = lane; i < dim; i += 64) {
-                const float a = x[i];
+                const float a = bias ? x[i] + bias[i] : x[i];
                 buf[i] = a;
                 ss += a * a;
             }
@@ -200,7 +201,8 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
     const float slope = p.slopes ? p.slopes[h] : 0.f;
     const bool sig = p.pb != nullptr;
     const float pbh = sig ? p.pb[h] : 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    // a sink is a score without key or value: the running maximum and sum start from it
+    float m_run = p.sink ? p.sink[h] : -INFINITY, l_run = p.sink ? 1.f : 0.f;
     float acc[GA_MAXV] = {};
     for (int j0 = lo; j0 <= pos; j0 += GA_CHUNK) {
         const int nk = min(GA_CHUNK, pos + 1 - j0);
@@ -272,11 +274,15 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
         __syncthreads();
     }
     float inv = sig ? 1.0f : 1.0f / l_run;
-    if (p.gate_col >= 0) inv *= 1.0f / (1.0f + expf(-p.proj[(int64_t)t * p.ld + p.gate_col + h]));
+    if (p.gate_col >= 0 && !p.gate_elem) inv *= 1.0f / (1.0f + expf(-p.proj[(int64_t)t * p.ld + p.gate_col + h]));
 #pragma unroll
     for (int i = 0; i < GA_MAXV; i++) {
         const int r = tid + i * 256;
-        if (r < vdim) ob[r] = acc[i] * inv;
+        if (r < vdim) {
+            float o = acc[i] * inv;
+            if (p.gate_col >= 0 && p.gate_elem) o *= 1.0f / (1.0f + expf(-p.proj[(int64_t)t * p.ld + p.gate_col + h * vdim + r]));
+            ob[r] = o;
+        }
     }
     __syncthreads();
     const float* vcs = p.rot_values ? p.vrope_cos + (int64_t)pos * (vdim / 2) : nullptr;
@@ -365,7 +371,8 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const float y = o[j] * a.out_scale;
+            float y = o[j] * a.out_scale;
+            if (a.gate_col >= 0 && a.gate_elem) y *= 1.0f / (1.0f + __expf(-a.proj[(int64_t)row * a.ld + a.gate_col + hh * vdim + v0 + j]));
             a.out[o0 + v0 + j] = y;
             if (a.out_bf) a.out_bf[o0 + v0 + j] = f2bf(y);
         }
@@ -374,9 +381,11 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
 
 // What a column's value sums are multiplied by: 1 / (sum of its softmax weights), or 1 for sigmoid
 // weights; times the head's sigmoid gate when the mixer has one.
-__device__ __forceinline__ float gqa_out_factor(const GqaAttnP& a, float l, int row, int hh) {
+// (m: the maximum the weights were taken against; a sink joins the sum as exp(sink_h - m))
+__device__ __forceinline__ float gqa_out_factor(const GqaAttnP& a, float l, float m, int row, int hh) {
+    if (a.sink) l += __expf(a.sink[hh] - m);
     float f = a.pb ? 1.0f : 1.0f / l;
-    if (a.gate_col >= 0) f *= 1.0f / (1.0f + __expf(-a.proj[(int64_t)row * a.ld + a.gate_col + hh]));
+    if (a.gate_col >= 0 && !a.gate_elem) f *= 1.0f / (1.0f + __expf(-a.proj[(int64_t)row * a.ld + a.gate_col + hh]));
     return f;
 }
 
@@ -568,7 +577,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
     }
     if (!active) return;
     if (S == 1) {
-        if (valid) gqa_store<DV>(a, acc, gqa_out_factor(a, l_run, row, hh), row, hh, qpos, g);
+        if (valid) gqa_store<DV>(a, acc, gqa_out_factor(a, l_run, m_run, row, hh), row, hh, qpos, g);
         return;
     }
     const int64_t unit = ((int64_t)blockIdx.x * (gridDim.y * 4) + tile) * S + z;
@@ -625,7 +634,7 @@ __global__ __launch_bounds__(256) void gqa_attn_combine_kernel(GqaAttnMfmaP P, i
             acc[dv][3] += o0[dv].w * w0 + o1[dv].w * w1;
         }
     }
-    gqa_store<DV>(a, acc, gqa_out_factor(a, L, grp.x + tI, hh), grp.x + tI, hh, pos0 + tI, g);
+    gqa_store<DV>(a, acc, gqa_out_factor(a, L, M, grp.x + tI, hh), grp.x + tI, hh, pos0 + tI, g);
 }
 
 bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens) {
@@ -921,7 +930,7 @@ int mingru_carry(const MinGruCarryP& p, hipStream_t st) {
 // ------------------------------------------------------------------ per-head norm
 __global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, const float* o2, const float* w, float eps, float scale,
                                                              int heads, int vdim, float* out, uint16_t* out_bf, int64_t ld_out,
-                                                             int out_col) {
+                                                             int out_col, const float* gate) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int h = wave; h < heads; h += 4) {
@@ -936,16 +945,17 @@ __global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, con
         const float inv = scale / sqrtf(ss / (float)vdim + eps);
         const int64_t o0 = t * ld_out + out_col + (int64_t)h * vdim;
         for (int i = lane; i < vdim; i += 64) {
-            const float y = (x2 ? x[i] + x2[i] : x[i]) * inv * w[i];
+            float y = (x2 ? x[i] + x2[i] : x[i]) * inv * w[i];
+            if (gate) y *= 1.0f / (1.0f + expf(-gate[(t * heads + h) * vdim + i]));
             out[o0 + i] = y;
             if (out_bf) out_bf[o0 + i] = f2bf(y);
         }
     }
 }
 int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
-                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st) {
+                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st, const float* gate) {
     hipLaunchKernelGGL(head_norm_rows_kernel, dim3(T), dim3(256), 0, st, o, o2, w, eps, scale, heads, vdim, out, out_bf, ld_out,
-                       out_col);
+                       out_col, gate);
     QIE_LAUNCH_CHECK();
     return 0;
 }

@@ -171,7 +171,8 @@ def tp_shardable(spec: ModelSpec, tp: int):
 
 @dataclasses.dataclass(frozen=True)
 class LatentAttention:
-    """Mixer: latent (compressed-KV) attention over a sliding window with a per-head output gate."""
+    """Mixer: latent (compressed-KV) attention, causal or over a sliding window; options: a per-head
+    output gate, queries through a latent of their own, either rotary pairing, scaled frequencies."""
     heads: int
     dim: int          # unrotated query / key coordinates per head
     rot_dim: int      # rotated coordinates per head (the key's are shared by all heads)
@@ -182,6 +183,10 @@ class LatentAttention:
     rot_base: float
     scale: float
     kv_from: Optional[int] = None   # the layer whose cache rows this layer reads
+    q_rank: int = 0                 # > 0: q = W_uq rms(W_dq x) w through a latent of this size (no W_q)
+    rot_layout: str = "halves"      # "halves" | "interleaved"
+    head_gate: bool = True          # head h's output times sigmoid(W_g x)_h
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None   # (factor, low, high, original)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -208,6 +213,10 @@ class GqaAttention:
     head_gate: bool = False      # head h's output times sigmoid(W_g x)_h
     q_temp_coef: float = 0.0     # q times 1 + coef * ln(floor((pos + 1) / every) + 1) after its norm
     q_temp_every: int = 0        # 0: no query temperature
+    qk_bias: bool = False        # bias vectors on the q and k projections
+    sink: bool = False           # exp(a number per head) joins the softmax denominator
+    out_gate: bool = False       # the concatenated head outputs times sigmoid(W_g x), element by element
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None   # (factor, low, high, original) wavelengths
 
 
 @dataclasses.dataclass(frozen=True)
@@ -236,6 +245,23 @@ class MinGru:
 
 
 @dataclasses.dataclass(frozen=True)
+class ChannelDelta:
+    """Mixer: gated delta rule with one decay per head and key channel; short convolutions on q, k, v;
+    a [dim, vdim] fp32 state per head and slot plus the convolutions' last inputs."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int         # taps of the short convolutions
+    rank_a: int       # rows of W_a1 (decay) and W_g1 (output gate)
+    rank_g: int
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+
+@dataclasses.dataclass(frozen=True)
 class FeedForward:
     kind: str         # "dense" or "moe"
     ff: int           # hidden size (of one expert for "moe")
@@ -245,7 +271,7 @@ class FeedForward:
                                  # biased logits, softmax over the chosen ones weights the output;
                                  # "softmax_all": softmax over all router outputs, chosen by score +
                                  # correction inside the best groups, renormalised, times route_scale
-    act: str = "silu_gated"      # dense: "silu_gated" (gate, up, down) | "xielu" (up, down, two numbers)
+    act: str = "silu_gated"      # dense: "silu_gated" | "gelu_tanh_gated" (gate, up, down) | "xielu" (up, down, two numbers)
     identity: int = 0            # "softmax_all": identity experts after the `experts` real ones
     groups: int = 1
     groups_keep: int = 1
@@ -254,7 +280,7 @@ class FeedForward:
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    mixer: object     # LatentAttention | GqaAttention | AttentionWithRecurrence | MinGru
+    mixer: object     # LatentAttention | GqaAttention | AttentionWithRecurrence | MinGru | ChannelDelta
     mlp: Optional[FeedForward]
 
 
@@ -272,6 +298,11 @@ class LayeredSpec:
     embed_scale: float = 1.0
     pos_embed: str = "none"          # "none" | "sinusoid" (added to the scaled embedding row)
     loop: Optional[Tuple[int, int, int]] = None   # (start, stop, times): layers [start, stop) run `times` times
+    # pre-norm block options
+    norm_offset: float = 0.0         # norm weights are norm_offset + w (1: stored around zero)
+    streams: int = 0                 # >= 1: that many residual rows mixed by 'l<i>.hc<q>.in|out|mix' (hyper-connections)
+    canon_taps: int = 0              # >= 1: the mixer reads h + causal conv(h) over time ('l<i>.canon1' [width, taps])
+    embed_norm: bool = False         # the embedding rows are normed with 'embed.norm'
 
     @property
     def n_layers(self) -> int:
@@ -307,6 +338,9 @@ class LayeredSpec:
             g.weights = _lib.QIE_WEIGHTS_SIGMOID if m.weights == "sigmoid" else _lib.QIE_WEIGHTS_SOFTMAX
             g.slope_bias, g.head_gate = int(m.slope_bias), int(m.head_gate)
             g.q_temp_coef, g.q_temp_every = m.q_temp_coef, m.q_temp_every
+            g.qk_bias, g.sink, g.out_gate = int(m.qk_bias), int(m.sink), int(m.out_gate)
+            if m.rot_scaling:
+                g.rot_scaling.factor, g.rot_scaling.low, g.rot_scaling.high, g.rot_scaling.original = m.rot_scaling
 
         for d, L in zip(arr, self.layers):
             m = L.mixer
@@ -321,16 +355,25 @@ class LayeredSpec:
             elif isinstance(m, MinGru):
                 d.mixer = _lib.QIE_MIXER_MINGRU
                 d.mingru.width = m.width
+            elif isinstance(m, ChannelDelta):
+                d.mixer = _lib.QIE_MIXER_CHANNEL_DELTA
+                x = d.delta
+                x.heads, x.kv_heads, x.dim, x.vdim, x.conv, x.rank_a, x.rank_g = m.heads, m.kv_heads, m.dim, m.vdim, m.conv, m.rank_a, m.rank_g
             else:
                 d.mixer = _lib.QIE_MIXER_LATENT_ATTENTION
                 d.heads, d.dim, d.rot_dim, d.vdim, d.kv_rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
                 d.window, d.kv_from, d.rot_dims = m.window, -1 if m.kv_from is None else m.kv_from, m.rot_dims
                 d.rot_base, d.scale = m.rot_base, m.scale
+                d.q_rank, d.head_gate = m.q_rank, int(m.head_gate)
+                d.rot_layout = {"halves": _lib.QIE_ROT_HALVES, "interleaved": _lib.QIE_ROT_INTERLEAVED}[m.rot_layout]
+                if m.rot_scaling:
+                    d.rot_scaling.factor, d.rot_scaling.low, d.rot_scaling.high, d.rot_scaling.original = m.rot_scaling
             if L.mlp is None:
                 d.ff_kind = _lib.QIE_FF_NONE
             elif L.mlp.kind == "dense":
                 d.ff_kind, d.ff = _lib.QIE_FF_DENSE, L.mlp.ff
-                d.ff_act = _lib.QIE_ACT_XIELU if L.mlp.act == "xielu" else _lib.QIE_ACT_SILU_GATED
+                d.ff_act = {"silu_gated": _lib.QIE_ACT_SILU_GATED, "xielu": _lib.QIE_ACT_XIELU,
+                            "gelu_tanh_gated": _lib.QIE_ACT_GELU_TANH_GATED}[L.mlp.act]
             else:
                 d.ff_kind, d.ff, d.experts, d.top = _lib.QIE_FF_MOE, L.mlp.ff, L.mlp.experts, L.mlp.top
                 d.router = {"sigmoid_in": _lib.QIE_ROUTER_SIGMOID_IN, "softmax_out": _lib.QIE_ROUTER_SOFTMAX_OUT,
@@ -347,6 +390,7 @@ class LayeredSpec:
         if self.loop:
             a.loop_start, a.loop_stop, a.loop_times = self.loop
         a.layers = arr
+        a.streams, a.canon_taps, a.embed_norm, a.norm_offset = self.streams, self.canon_taps, int(self.embed_norm), self.norm_offset
         return a, arr
 
     def tensor_shapes(self) -> "dict[str, List[int]]":
@@ -367,10 +411,22 @@ class LayeredSpec:
                 out[q + "pb"] = [m.heads]
             if m.head_gate:
                 out[q + "g"] = [m.heads, W]
+            if m.qk_bias:
+                out[q + "q.b"], out[q + "k.b"] = [m.heads * m.dim], [m.kv_heads * m.dim]
+            if m.sink:
+                out[q + "sink"] = [m.heads]
+            if m.out_gate:
+                out[q + "g"] = [m.heads * m.vdim, W]
             out[q + "o"] = [W, m.heads * m.vdim]
 
+        if self.embed_norm:
+            out["embed.norm"] = [W]
         for i, L in enumerate(self.layers):
             m, p = L.mixer, f"l{i}."
+            for q in (("hc1.", "hc2.") if L.mlp is not None else ("hc1.",)) if self.streams else ():
+                out[p + q + "in"], out[p + q + "out"], out[p + q + "mix"] = [self.streams], [self.streams], [self.streams, self.streams]
+            if self.canon_taps:
+                out[p + "canon1"] = [W, self.canon_taps]
             out[p + "norm1"] = nshape
             if sandwich:
                 out[p + "norm1b"] = nshape
@@ -390,14 +446,26 @@ class LayeredSpec:
                 q = p + "mix."
                 out.update({q + "z": [m.width, W], q + "z.b": [m.width], q + "x": [m.width, W], q + "x.b": [m.width],
                             q + "g": [m.width, W], q + "o": [W, m.width]})
+            elif isinstance(m, ChannelDelta):
+                q = p + "mix."
+                nk, nv = m.kv_heads * m.dim, m.heads * m.vdim
+                out.update({q + "q": [nk, W], q + "q.conv": [nk, m.conv], q + "k": [nk, W], q + "k.conv": [nk, m.conv],
+                            q + "v": [nv, W], q + "v.conv": [nv, m.conv], q + "b": [m.heads, W], q + "A_log": [m.heads],
+                            q + "norm": [m.vdim], q + "a1": [m.rank_a, W], q + "a2": [m.heads * m.dim, m.rank_a],
+                            q + "dt_bias": [m.heads * m.dim], q + "g1": [m.rank_g, W], q + "g2": [nv, m.rank_g], q + "o": [W, nv]})
+            elif m.q_rank > 0:
+                out[p + "mix.dq"], out[p + "mix.dq.norm"] = [m.q_rank, W], [m.q_rank]
+                out[p + "mix.uq"] = [m.heads * (m.dim + m.rot_dim), m.q_rank]
             else:
                 out[p + "mix.q"] = [m.heads * (m.dim + m.rot_dim), W]
+            if isinstance(m, LatentAttention):
                 if m.kv_from is None:
                     out[p + "mix.dkv"] = [m.kv_rank + m.rot_dim, W]
                     out[p + "mix.dkv.norm"] = [m.kv_rank]
                 out[p + "mix.uk"] = [m.heads * m.dim, m.kv_rank]
                 out[p + "mix.uv"] = [m.heads * m.vdim, m.kv_rank]
-                out[p + "mix.g"] = [m.heads, W]
+                if m.head_gate:
+                    out[p + "mix.g"] = [m.heads, W]
                 out[p + "mix.o"] = [W, m.heads * m.vdim]
             if L.mlp is not None and L.mlp.kind == "dense" and L.mlp.act == "xielu":
                 out.update({p + "mlp.up": [L.mlp.ff, W], p + "mlp.down": [W, L.mlp.ff], p + "mlp.act": [2]})
@@ -426,7 +494,7 @@ class LayeredSpec:
             m = self.layers[i].mixer
             if isinstance(m, LatentAttention):
                 n += m.kv_rank + m.rot_dim if m.kv_from is None else 0
-            elif isinstance(m, MinGru):
+            elif isinstance(m, (MinGru, ChannelDelta)):
                 pass
             else:
                 a = m.attn if isinstance(m, AttentionWithRecurrence) else m
@@ -442,6 +510,10 @@ class LayeredSpec:
                 n += m.rec.heads * m.rec.dim * m.rec.vdim
             elif isinstance(m, MinGru):
                 n += m.width
+            elif isinstance(m, ChannelDelta):
+                n += m.heads * m.dim * m.vdim + (m.conv - 1) * m.conv_channels
+            if self.canon_taps > 1:
+                n += (self.canon_taps - 1) * self.width
         return n
 
     def step_flops(self, rows: int, ctx: int) -> float:
@@ -450,6 +522,13 @@ class LayeredSpec:
         for i in self.runs():
             L = self.layers[i]
             m = L.mixer
+            if isinstance(m, ChannelDelta):
+                nk, nv = m.kv_heads * m.dim, m.heads * m.vdim
+                f += 2.0 * rows * W * (2 * nk + 2 * nv + m.heads + m.rank_a + m.rank_g)
+                f += 2.0 * rows * (m.rank_a * m.heads * m.dim + m.rank_g * nv) + 2.0 * rows * m.heads * m.dim * m.vdim * 3
+                if L.mlp is not None:
+                    f += 2.0 * rows * 3 * W * L.mlp.ff
+                continue
             if isinstance(m, MinGru):
                 f += 2.0 * rows * W * 4 * m.width
                 if L.mlp is not None:
@@ -457,7 +536,8 @@ class LayeredSpec:
                 continue
             if not isinstance(m, LatentAttention):
                 a = m.attn if isinstance(m, AttentionWithRecurrence) else m
-                n_in = a.heads * a.dim + a.kv_heads * (a.dim + (0 if a.values_are_keys else a.vdim)) + (a.heads if a.head_gate else 0)
+                n_in = a.heads * a.dim + a.kv_heads * (a.dim + (0 if a.values_are_keys else a.vdim)) + (a.heads if a.head_gate else 0) \
+                    + (a.heads * a.vdim if a.out_gate else 0)
                 n_cat = a.heads * a.vdim
                 keys = ctx if a.mask == "causal" else min(ctx, a.mask_size if a.mask == "window" else (a.mask_size + 1) // 2)
                 f += 2.0 * rows * a.heads * keys * (a.dim + a.vdim)
@@ -470,9 +550,11 @@ class LayeredSpec:
                 if L.mlp is not None:
                     f += 2.0 * rows * (1 if L.mlp.kind == "dense" else L.mlp.top) * (2 if L.mlp.act == "xielu" else 3) * W * L.mlp.ff
                 continue
-            n_in = m.heads * (m.dim + m.rot_dim) + m.heads + (m.kv_rank + m.rot_dim if m.kv_from is None else 0)
+            n_in = (m.heads * (m.dim + m.rot_dim) if m.q_rank == 0 else m.q_rank) + (m.heads if m.head_gate else 0) \
+                + (m.kv_rank + m.rot_dim if m.kv_from is None else 0)
+            f += 2.0 * rows * m.q_rank * m.heads * (m.dim + m.rot_dim)
             f += 2.0 * rows * W * n_in + 2.0 * rows * m.heads * m.kv_rank * (m.dim + m.vdim) + 2.0 * rows * W * m.heads * m.vdim
-            f += 2.0 * rows * m.heads * min(ctx, m.window) * (2 * m.kv_rank + m.rot_dim)
+            f += 2.0 * rows * m.heads * (min(ctx, m.window) if m.window > 0 else ctx) * (2 * m.kv_rank + m.rot_dim)
             if L.mlp is not None:
                 k = 1 if L.mlp.kind == "dense" else L.mlp.top
                 f += 2.0 * rows * k * 3 * W * L.mlp.ff
@@ -586,7 +668,66 @@ def _lugipel_from_config(cfg: dict, name: str) -> LayeredSpec:
                        pos_embed="sinusoid")
 
 
-ARCHITECTURES = {"Tivazen": _tivazen_from_config, "Nodutar": _nodutar_from_config, "Lugipel": _lugipel_from_config}
+def _rot_scaling(rot: dict):
+    sc = rot.get("scaling")
+    if not sc:
+        return None
+    t = (float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
+    if not (t[0] > 0 and t[2] > t[1] >= 0 and t[3] > 0):
+        raise ValueError(f"rotary scaling {sc}: factor and original must be positive, high above low")
+    return t
+
+
+def _verelorn_from_config(cfg: dict, name: str) -> LayeredSpec:
+    """Verelorn: pre-normed blocks (RMS norms with weights stored around zero, also on the embedding rows)
+    over several residual streams mixed by learned hyper-connections; the mixer reads its normed input
+    plus a short causal convolution of it.  Mixers: a causal grouped-query attention whose values are
+    its keys as projected (biased q / k, partial rotate-half rotary with wavelength-scaled frequencies,
+    a sink in the softmax, an element-wise sigmoid output gate); a latent attention with queries
+    through a latent of their own and an interleaved rotary on the shared key part, optionally reading
+    an earlier layer's cache; a gated delta rule with channel-wise decay.  Feed-forward: dense, gated
+    tanh-GELU, or none.  Untied head."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m = L["mixer"]
+        rot = m.get("rot") or {}
+        if L["type"] == "attention":
+            mixer = GqaAttention(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]),
+                rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), rot_layout="halves", mask="causal",
+                values_are_keys=True, qk_bias=True, sink=True, out_gate=True, rot_scaling=_rot_scaling(rot))
+            if mixer.vdim != mixer.dim:
+                raise ValueError(f"layer {i}: the values are the keys, so vdim {mixer.vdim} must equal dim {mixer.dim}")
+        elif L["type"] == "latent_attention":
+            mixer = LatentAttention(
+                heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+                window=0, rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)), scale=float(m["scale"]),
+                kv_from=None if m.get("kv_from") is None else int(m["kv_from"]), q_rank=int(m["q_rank"]), rot_layout="interleaved",
+                head_gate=False, rot_scaling=_rot_scaling(rot))
+        elif L["type"] == "channel_delta":
+            # the ranks of the decay and gate projections are sizes only the tensors give (0: taken from them)
+            mixer = ChannelDelta(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                 conv=int(m["conv"]), rank_a=int(m.get("rank_a", 0)), rank_g=int(m.get("rank_g", 0)))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        f = L.get("mlp")
+        if f is None:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForward("dense", int(f["ff"]), act="gelu_tanh_gated")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    streams = int(cfg.get("streams") or 0)
+    taps = int((cfg.get("canon") or {}).get("taps", 0))
+    if streams < 0 or streams > 8:
+        raise ValueError(f"streams {streams}: at most 8 residual streams")
+    return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), depth_mix=False,
+                       block="prenorm", tied_head=False, norm_offset=1.0, streams=streams, canon_taps=taps, embed_norm=True)
+
+
+ARCHITECTURES = {"Tivazen": _tivazen_from_config, "Nodutar": _nodutar_from_config, "Lugipel": _lugipel_from_config,
+                 "Verelorn": _verelorn_from_config}
 
 
 def spec_from_config(cfg: dict, name: str = "model", numerics: str = "hf"):
@@ -600,7 +741,32 @@ def spec_from_config(cfg: dict, name: str = "model", numerics: str = "hf"):
     return ModelSpec.from_hf_config(cfg, name=name, numerics=numerics)
 
 
+def with_tensor_sizes(spec, shapes: "dict[str, List[int]]"):
+    """Sizes a config leaves to the checkpoint's tensors (the ranks of a ChannelDelta's decay and gate
+    projections), filled in from a name -> shape table."""
+    if not isinstance(spec, LayeredSpec):
+        return spec
+    layers = list(spec.layers)
+    for i, L in enumerate(layers):
+        m = L.mixer
+        if isinstance(m, ChannelDelta) and (m.rank_a == 0 or m.rank_g == 0):
+            a1, g1 = shapes.get(f"l{i}.mix.a1"), shapes.get(f"l{i}.mix.g1")
+            if a1 is None or g1 is None:
+                raise ValueError(f"layer {i}: tensors 'l{i}.mix.a1' / 'l{i}.mix.g1' are missing")
+            layers[i] = LayerSpec(dataclasses.replace(m, rank_a=m.rank_a or int(a1[0]), rank_g=m.rank_g or int(g1[0])), L.mlp)
+    return dataclasses.replace(spec, layers=tuple(layers))
+
+
 def spec_from_dir(path: str, numerics: str = "hf"):
     import os
     with open(os.path.join(path, "config.json")) as f:
-        return spec_from_config(json.load(f), name=os.path.basename(os.path.normpath(path)), numerics=numerics)
+        spec = spec_from_config(json.load(f), name=os.path.basename(os.path.normpath(path)), numerics=numerics)
+    st = os.path.join(path, "model.safetensors")
+    if isinstance(spec, LayeredSpec) and os.path.exists(st) and any(
+            isinstance(L.mixer, ChannelDelta) and 0 in (L.mixer.rank_a, L.mixer.rank_g) for L in spec.layers):
+        import struct
+        with open(st, "rb") as f:
+            n = struct.unpack("<Q", f.read(8))[0]
+            hdr = json.loads(f.read(n))
+        spec = with_tensor_sizes(spec, {k: v["shape"] for k, v in hdr.items() if k != "__metadata__"})
+    return spec
