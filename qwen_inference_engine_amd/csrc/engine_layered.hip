@@ -146,7 +146,10 @@ struct LayeredBatch {
     float *s_loc = nullptr, *s_in = nullptr, *s_decay = nullptr;
     int64_t scan_cap = 0;             // pieces the three buffers hold
     int64_t m_state = 0, m_hd = 0;    // largest state / gate row count of a layer run
-    bool v_transposed = false;        // bf16 K / V caches on the matrix-core attention: V rows stored [kv_heads][vdim][page_tokens]
+    // bf16 K / V caches on the matrix-core attention: V rows stored [kv_heads][vdim][page_tokens].  Per layer run
+    // (vt_of): a grouped-query mixer whose sizes fit that kernel; v_transposed: any run does.
+    bool v_transposed = false;
+    std::vector<char> vt_of;
     float *gpart_o = nullptr, *gpart_ml = nullptr;   // its key-split partials
     int64_t gpart_cap = 0;            // (group, tile, split) units they hold
     int64_t cap = 0, want_cap = 0;
@@ -166,7 +169,10 @@ struct LayeredBatch {
     std::vector<int4> h_groups;
     float *part_o = nullptr, *part_ml = nullptr;
     int64_t part_cap = 0;         // (group, split) units the partials hold
-    bool interleaved = false;     // the cache pages carry the key-interleaved copy of c
+    // the cache pages carry the key-interleaved copy of c: per layer (il_of; a borrowing layer follows the layer
+    // whose rows it reads), interleaved: any layer does
+    bool interleaved = false;
+    std::vector<char> il_of;
     // per-expert products of prompt-sized steps run on side streams beside the engine's (every
     // expert's GEMM alone covers a fraction of the chip); default priority, joined by events
     static constexpr int kSide = 3;
@@ -743,7 +749,7 @@ static int enq_latent_post(qie_batch* b, int i, int T) {
     p.rope_sin = m->ropes[L.rope].sn;
     p.cache = cache_of(b);
     p.layer_off = s->layer_off[L.cache_layer];   // engines with latent layers run every layer once: run == layer
-    p.interleaved = s->interleaved;
+    p.interleaved = s->il_of[L.cache_layer];
     p.rot_layout = d.rot_layout;
     if (d.q_rank > 0 && p.own_kv) {   // the first-stage product holds [latent queries | compressed row | shared key part]
         p.kv = s->pre + d.q_rank;
@@ -782,7 +788,7 @@ static int enq_attention(qie_batch* b, int i, int T) {
     p.layer_off = s->layer_off[L.cache_layer];
     p.out = s->olat;
     auto it = s->groups.find(d.heads);
-    if (s->interleaved && it != s->groups.end() && lay::latent_attention_mfma_fits(d.kv_rank, d.rot_dim)) {
+    if (s->il_of[L.cache_layer] && it != s->groups.end() && lay::latent_attention_mfma_fits(d.kv_rank, d.rot_dim)) {
         // bf16 cache rows: the matrix-core kernel; enough key splits to fill the chip when the
         // step has few rows (decoding)
         const int ng = it->second.first;
@@ -830,7 +836,7 @@ static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
     const int pad = lay::kLatentQG;
     for (const LayerDev& L : m->L) {
         const int H = L.d.heads;
-        if (s->groups.count(H)) continue;
+        if (L.d.mixer != QIE_MIXER_LATENT_ATTENTION || !s->il_of[L.cache_layer] || s->groups.count(H)) continue;
         const int64_t first = (int64_t)s->h_groups.size();
         int row = 0;
         for (int i = 0; i < n_entries; i++) {
@@ -981,7 +987,7 @@ static lay::GqaAttnP gqa_attn_params(qie_batch* b, int r) {
     p.cache = cache_of(b);
     p.k_off = s->layer_off[r];
     p.v_off = s->v_off[r];
-    p.v_transposed = s->v_transposed;
+    p.v_transposed = s->vt_of[r];
     p.out_scale = L.d.mixer == QIE_MIXER_GQA_RECURRENT ? L.d.gqa_scale : 1.0f;
     p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = L.n_cat; p.out_col = 0;
     p.slopes = a.slope_bias ? L.slopes : nullptr;
@@ -1023,7 +1029,7 @@ static int enq_gqa_post(qie_batch* b, int r, int T) {
     p.cache = cache_of(b);
     p.k_off = s->layer_off[r];
     p.v_off = s->v_off[r];
-    p.v_transposed = s->v_transposed;
+    p.v_transposed = s->vt_of[r];
     p.q_temp_every = a.q_temp_every;
     p.q_temp_coef = a.q_temp_coef;
     p.q_bias = a.qk_bias ? L.q_bias : nullptr;
@@ -1035,7 +1041,7 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
     const qie_engine* e = b->e;
     LayeredBatch* s = b->lb;
     const lay::GqaAttnP p = gqa_attn_params(b, r);
-    if (s->v_transposed && s->n_qgroups > 0) {
+    if (p.v_transposed && s->n_qgroups > 0) {
         // enough key splits to fill the chip when the step has few rows (decoding)
         const int tiles = (p.heads + 3) / 4 * 4;
         const int64_t waves = (int64_t)s->n_qgroups * p.heads;
@@ -1599,19 +1605,24 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     s->canon_off.assign(n_runs, 0);
     // bf16 caches whose every layer fits the matrix-core attention carry, after the rows of a
     // caching layer, the key-interleaved copy of c (R more elements per token)
-    s->interleaved = !m->f32;
-    for (int i = 0; i < m->a.n_layers; i++)
-        if (m->L[i].d.mixer != QIE_MIXER_LATENT_ATTENTION ||
-            !lay::latent_attention_mfma_fits(m->L[i].d.kv_rank, m->L[i].d.rot_dim))
-            s->interleaved = false;
-    // bf16 grouped-query caches whose every layer fits the matrix-core attention store V transposed
-    s->v_transposed = !m->f32;
+    s->il_of.assign(m->a.n_layers, 0);
     for (int i = 0; i < m->a.n_layers; i++) {
         const qie_layer_desc& d = m->L[i].d;
-        if (d.mixer == QIE_MIXER_MINGRU || d.mixer == QIE_MIXER_CHANNEL_DELTA) continue;   // cache nothing
-        if (d.mixer == QIE_MIXER_LATENT_ATTENTION || !lay::gqa_attention_mfma_fits(d.gqa.dim, d.gqa.vdim, page_tokens))
-            s->v_transposed = false;
-        if (d.mixer != QIE_MIXER_LATENT_ATTENTION) s->m_vd = std::max<int64_t>(s->m_vd, d.gqa.vdim);
+        if (!m->f32 && d.mixer == QIE_MIXER_LATENT_ATTENTION && page_tokens % 16 == 0 &&
+            lay::latent_attention_mfma_fits(d.kv_rank, d.rot_dim))
+            s->il_of[i] = 1;
+    }
+    for (int i = 0; i < m->a.n_layers; i++) {
+        if (m->L[i].d.mixer == QIE_MIXER_LATENT_ATTENTION) s->il_of[i] = s->il_of[m->L[i].cache_layer];
+        if (s->il_of[i]) s->interleaved = true;
+    }
+    // bf16 grouped-query caches whose every layer fits the matrix-core attention store V transposed
+    s->vt_of.assign(n_runs, 0);
+    for (int r = 0; r < n_runs; r++) {
+        const qie_layer_desc& d = m->L[m->runs[r].layer].d;
+        if (d.mixer != QIE_MIXER_GQA && d.mixer != QIE_MIXER_GQA_RECURRENT) continue;
+        if (!m->f32 && lay::gqa_attention_mfma_fits(d.gqa.dim, d.gqa.vdim, page_tokens)) s->vt_of[r] = 1, s->v_transposed = true;
+        s->m_vd = std::max<int64_t>(s->m_vd, d.gqa.vdim);
     }
     int64_t off = 0;
     for (int r = 0; r < n_runs; r++) {
@@ -1682,7 +1693,7 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
         }
         if (d.kv_from < 0) {
             s->layer_off[i] = off;
-            off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim + (s->interleaved ? d.kv_rank : 0));
+            off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim + (s->il_of[i] ? d.kv_rank : 0));
         }
         const int64_t H = d.heads;
         s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);

@@ -21,7 +21,7 @@ def pytest_collection_modifyitems(config, items):
     on different hardware queues, and which queue a new stream gets depends on how many streams the
     process has created before.  Those tests were written under the stream history of the modules
     before them; modules that create many engines of their own therefore go last."""
-    names = ("test_gpu_layered", "test_gpu_nodutar", "test_gpu_lugipel")
+    names = ("test_gpu_layered", "test_gpu_nodutar", "test_gpu_lugipel", "test_gpu_verelorn")
     late = [it for it in items if any(n in it.nodeid for n in names)]
     if late:
         items[:] = [it for it in items if not any(n in it.nodeid for n in names)] + late

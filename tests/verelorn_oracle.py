@@ -246,3 +246,104 @@ def forward(cfg, W, tokens, layers_out=None):
             layers_out.append(X.sum(axis=0))
     x = norm_offset(X.sum(axis=0), W["final.norm"], eps)
     return x @ f64(W["head"]).T
+
+
+# ---------------------------------------------------------------- small configurations and random weights
+def dense(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def attn(heads=4, kv_heads=2, dim=16, rot_dims=8, base=10000.0, scaling=None, scale=None, mlp="dense"):
+    rot = {"base": base, "dims": rot_dims}
+    if scaling:
+        rot["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale if scale is not None else dim ** -0.5}
+    if rot_dims:
+        m["rot"] = rot
+    return {"type": "attention", "mixer": m, "mlp": dense() if mlp == "dense" else mlp}
+
+
+def latent(heads=2, dim=8, rot_dim=4, vdim=12, kv_rank=16, q_rank=24, base=10000.0, kv_from=None, scale=None, mlp="dense"):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "rot": {"base": base, "dims": rot_dim}, "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m, "mlp": dense() if mlp == "dense" else mlp}
+
+
+def delta(heads=2, kv_heads=1, dim=8, vdim=12, conv=3, ranks=(6, 5), mlp=None):
+    """ranks: rows of a1 / g1 - sizes only the tensors carry."""
+    return {"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv},
+            "mlp": dense() if mlp == "dense" else mlp, "_ranks": ranks}
+
+
+def config(layers, vocab=101, width=40, eps=1e-5, streams=3, taps=3):
+    cfg = {"architecture": "Verelorn", "vocab": vocab, "width": width, "norm": {"eps": eps},
+           "layers": [{k: v for k, v in L.items() if k != "_ranks"} for L in layers]}
+    if streams:
+        cfg["streams"] = streams
+    if taps:
+        cfg["canon"] = {"taps": taps}
+    cfg["_ranks"] = [L.get("_ranks") for L in layers]
+    return cfg
+
+
+def to_bf16_exact(a):
+    """float32 values rounded to the nearest bf16 (kept as float32)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & np.uint32(0xFFFF0000)
+    return u.view(np.float32).reshape(np.shape(a))
+
+
+def random_weights(cfg, seed=0, qk_gain=2.0):
+    """{name: float32 array of exact bf16 values} for a config made by config().  The branches' output projections
+    are small beside the residual rows, as in a trained model: a rounding error then shrinks from layer to layer
+    instead of doubling.  qk_gain: how sharp the softmaxes are (scores of a few units at 2, which a tight fp32
+    comparison wants; 1 for comparisons of bf16 engines, whose rounded keys move sharp weights by percents)."""
+    rng = np.random.default_rng(seed)
+    W, V, T = cfg["width"], cfg["vocab"], {}
+
+    def lin(o, i, gain=1.0):
+        return rng.normal(0.0, gain / math.sqrt(i), (o, i))
+
+    def vec(n, sd=0.2, mean=0.0):
+        return mean + rng.normal(0.0, sd, n)
+
+    T["embed"], T["embed.norm"], T["final.norm"], T["head"] = rng.normal(0, 1, (V, W)), vec(W), vec(W), lin(V, W)
+    n = int(cfg.get("streams") or 0)
+    taps = int((cfg.get("canon") or {}).get("taps", 0))
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        subs = (1, 2) if L.get("mlp") is not None else (1,)
+        for q in subs:
+            T[f"{p}norm{q}"] = vec(W)
+            if n:
+                T[f"{p}hc{q}.in"] = vec(n, 0.2, 1.0 / n)
+                T[f"{p}hc{q}.out"] = vec(n, 0.3, 0.7)
+                T[f"{p}hc{q}.mix"] = np.eye(n) * 0.8 + rng.normal(0, 0.15, (n, n))
+        if taps:
+            T[p + "canon1"] = rng.normal(0, 0.4, (W, taps))
+        x = p + "mix."
+        if L["type"] == "attention":
+            H, G, D = m["heads"], m["kv_heads"], m["dim"]
+            T[x + "q"], T[x + "k"], T[x + "g"], T[x + "o"] = lin(H * D, W, qk_gain), lin(G * D, W, qk_gain), lin(H * D, W), lin(W, H * D, 0.5)
+            T[x + "q.b"], T[x + "k.b"], T[x + "sink"] = vec(H * D, 0.5), vec(G * D, 0.5), vec(H, 1.0, 1.0)
+        elif L["type"] == "latent_attention":
+            H, D, Dr, Dv, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            T[x + "dq"], T[x + "dq.norm"], T[x + "uq"] = lin(Q, W), vec(Q, 0.2, 1.0), lin(H * (D + Dr), Q, qk_gain)
+            if m.get("kv_from") is None:
+                T[x + "dkv"], T[x + "dkv.norm"] = lin(R + Dr, W, qk_gain), vec(R, 0.2, 1.0)
+            T[x + "uk"], T[x + "uv"], T[x + "o"] = lin(H * D, R, qk_gain), lin(H * Dv, R), lin(W, H * Dv, 0.5)
+        else:
+            H, G, D, Dv, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+            ra, rg = cfg["_ranks"][i]
+            T[x + "q"], T[x + "k"], T[x + "v"], T[x + "b"] = lin(G * D, W, 2.0), lin(G * D, W, 2.0), lin(H * Dv, W, 2.0), lin(H, W, 2.0)
+            for t, c in (("q", G * D), ("k", G * D), ("v", H * Dv)):
+                T[f"{x}{t}.conv"] = rng.normal(0, 0.6, (c, K))
+            T[x + "A_log"], T[x + "dt_bias"], T[x + "norm"] = vec(H, 0.7, -1.0), vec(H * D, 1.0), vec(Dv, 0.2, 1.0)
+            T[x + "a1"], T[x + "a2"], T[x + "g1"], T[x + "g2"] = lin(ra, W), lin(H * D, ra, 2.0), lin(rg, W), lin(H * Dv, rg, 2.0)
+            T[x + "o"] = lin(W, H * Dv, 0.5)
+        if L.get("mlp") is not None:
+            ff = L["mlp"]["ff"]
+            T[p + "mlp.gate"], T[p + "mlp.up"], T[p + "mlp.down"] = lin(ff, W, 1.5), lin(ff, W), lin(W, ff, 0.5)
+    return {k: to_bf16_exact(v) for k, v in T.items()}
