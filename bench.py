@@ -74,6 +74,16 @@ LUGIPEL_SIZES = {
 }
 
 
+# Sizes of `--verelorn`: (width, attention heads, kv heads, head dim, rotated dims, latent heads, latent dim, latent
+# rot_dim, latent vdim, kv_rank, q_rank, delta heads, delta key heads, delta dim, delta vdim, delta taps, decay /
+# gate rank, ff, streams, input taps, vocab).  Four layers: latent attention + ff, sink attention + ff, delta rule
+# (no ff), latent attention on the first layer's cache + ff.
+VERELORN_SIZES = {
+    "1k": (1024, 16, 4, 64, 32, 16, 64, 32, 64, 256, 384, 16, 8, 64, 64, 4, 64, 2816, 4, 4, 32000),
+    "2k": (2048, 16, 4, 128, 64, 16, 128, 64, 128, 512, 768, 16, 8, 128, 128, 4, 64, 5632, 4, 4, 32000),
+}
+
+
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,6 +130,10 @@ def parse(argv=None):
                          "layers beside it (one JSON line of its own)")
     ap.add_argument("--lugipel", choices=sorted(LUGIPEL_SIZES), default=None,
                     help="instead of the default workload: prefill and decode throughput of a Lugipel model at this "
+                         "size with random weights, per-stage times, and the Qwen decoder at equal width / heads / "
+                         "layers beside it (one JSON line of its own)")
+    ap.add_argument("--verelorn", choices=sorted(VERELORN_SIZES), default=None,
+                    help="instead of the default workload: prefill and decode throughput of a Verelorn model at this "
                          "size with random weights, per-stage times, and the Qwen decoder at equal width / heads / "
                          "layers beside it (one JSON line of its own)")
     ap.add_argument("--dry-run", action="store_true",
@@ -181,6 +195,8 @@ def main(argv=None):
         return run_nodutar(a)
     if a.lugipel:
         return run_lugipel(a)
+    if a.verelorn:
+        return run_verelorn(a)
     return run(a)
 
 
@@ -455,6 +471,126 @@ def run_lugipel(a):
     eng.close()
     out["qwen_equal_size"] = qwen_twin(Q, S, Wt, a.lugipel, W, H, G, hd, 2 * top * eff, V, P, B, steps, prompts, a.prefill_iters,
                                        max_ctx)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def verelorn_model(S, size):
+    """(LayeredSpec, {name: bf16 words}) at one of VERELORN_SIZES, random weights from one pool."""
+    W, H, G, hd, rot, LH, ld, lr, lv, R, QR, DH, DG, dd, dv, taps_d, rank, ff, streams, taps, V = VERELORN_SIZES[size]
+    mlp = {"kind": "dense", "ff": ff}
+    lat = lambda kv_from: {"type": "latent_attention", "mlp": mlp, "mixer": dict(
+        {"heads": LH, "dim": ld, "rot_dim": lr, "vdim": lv, "kv_rank": R, "q_rank": QR, "rot": {"base": 1e6, "dims": lr},
+         "scale": (ld + lr) ** -0.5}, **({} if kv_from is None else {"kv_from": kv_from}))}
+    att = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+        "rot": {"base": 250000.0, "dims": rot, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 1024}}}}
+    dlt = {"type": "channel_delta", "mlp": None, "mixer": {"heads": DH, "kv_heads": DG, "dim": dd, "vdim": dv, "conv": taps_d}}
+    cfg = {"architecture": "Verelorn", "layers": [lat(None), att, dlt, lat(0)], "norm": {"eps": 1e-5}, "streams": streams,
+           "canon": {"taps": taps}, "vocab": V, "width": W}
+    spec = S.spec_from_config(cfg, name=f"verelorn-{size}")
+    spec = S.with_tensor_sizes(spec, {"l2.mix.a1": [rank, W], "l2.mix.g1": [rank, W]})
+    pool = np.random.default_rng(0).standard_normal(1 << 22).astype(np.float32)
+    tensors = {}
+    for k, (name, shape) in enumerate(spec.tensor_shapes().items()):
+        n = int(np.prod(shape))
+        if name.endswith(("dq.norm", "dkv.norm", "mix.norm", "hc1.out", "hc2.out")):
+            v = np.ones(shape, np.float32)
+        elif name.endswith(("norm1", "norm2", "final.norm", "embed.norm", "q.b", "k.b", "sink", "dt_bias")):
+            v = np.zeros(shape, np.float32)
+        elif name.endswith("A_log"):
+            v = np.full(shape, -1.0, np.float32)
+        elif name.endswith(("hc1.in", "hc2.in")):
+            v = np.full(shape, 1.0 / streams, np.float32)
+        elif name.endswith(("hc1.mix", "hc2.mix")):
+            v = np.eye(streams, dtype=np.float32)
+        else:
+            fan = shape[-1] if name != "embed" else 1
+            v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
+        tensors[name] = (np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
+    return spec, tensors
+
+
+def run_verelorn(a):
+    """Prefill (one step of P tokens) and decode (B single-token entries a step at context ~P) of a Verelorn model,
+    per-stage hipEvent times at both shapes, and the Qwen decoder at equal sizes."""
+    import qwen_inference_engine_amd as Q
+    from qwen_inference_engine_amd import spec as S, weights as Wt
+    W, H, G, hd, rot, LH, ld, lr, lv, R, QR, DH, DG, dd, dv, taps_d, rank, ff, streams, taps, V = VERELORN_SIZES[a.verelorn]
+    P, B, steps = a.prompt, max(a.batch, 8), min(a.steps, 128)
+    max_ctx = P + steps + 80
+    spec, tensors = verelorn_model(S, a.verelorn)
+    names = ("width", "heads", "kv_heads", "head_dim", "rot_dims", "latent_heads", "latent_dim", "latent_rot_dim", "latent_vdim",
+             "kv_rank", "q_rank", "delta_heads", "delta_kv_heads", "delta_dim", "delta_vdim", "delta_taps", "delta_rank", "ff",
+             "streams", "input_taps", "vocab")
+    out = {"metric": "verelorn_decode_tokens_per_sec", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights, random token ids)", "higher_is_better": True,
+           "config": {"model": spec.name, "sizes": dict(zip(names, VERELORN_SIZES[a.verelorn])), "layers": 4, "prompt": P,
+                      "decode_batch": B, "decode_steps": steps}}
+    eng = Q.Engine(spec, max_ctx=max_ctx).load_tensors(tensors)
+    del tensors
+    b = eng.batch(B, max_ctx, page_tokens=64)
+    rng = np.random.default_rng(1)
+    prompts = rng.integers(0, V, size=(B, P), dtype=np.int32)
+    ts = []
+    for it in range(1 + a.prefill_iters):
+        t0 = time.perf_counter()
+        b.step([(0, prompts[0])], [P - 1], fetch=False)
+        ts.append(time.perf_counter() - t0)
+        if it < a.prefill_iters:
+            b.release(0)
+    t_pf = float(np.median(ts[1:]))
+    stages = {"prefill": {}, "decode": {}}
+    C = 2 * DG * dd + DH * dv
+    att_in, lat_in = H * hd + G * hd + H * hd, QR + R + lr
+    dl_in = C + DH + 2 * rank
+
+    def stage_times(tag, rows, ctx):
+        st = stages[tag]
+        st["sink_attention_us"] = round(b.time_stage(1, 1, 10), 2)
+        st["latent_attention_us"] = round(b.time_stage(1, 0, 10), 2)
+        st["attention_products_us"] = round(b.time_stage(2, 1, 10), 2)
+        st["latent_products_us"] = round(b.time_stage(2, 0, 10), 2)
+        st["delta_products_us"] = round(b.time_stage(2, 2, 10), 2)
+        st["dense_ff_us"] = round(b.time_stage(3, 0, 10), 2)
+        st["delta_scan_us"] = round(b.time_stage(4, 2, 10), 2)
+        keys = ctx if tag == "decode" else ctx / 2.0
+        st["sink_attention_tflops"] = round(4.0 * rows * H * keys * hd / st["sink_attention_us"] / 1e6, 2)
+        st["latent_attention_tflops"] = round(2.0 * rows * LH * keys * (2 * R + lr) / st["latent_attention_us"] / 1e6, 2)
+        st["attention_products_tflops"] = round(2.0 * rows * W * (att_in + H * hd) / st["attention_products_us"] / 1e6, 2)
+        st["latent_products_tflops"] = round(2.0 * rows * (W * lat_in + QR * LH * (ld + lr) + LH * R * (ld + lv) + W * LH * lv) /
+                                             st["latent_products_us"] / 1e6, 2)
+        st["delta_products_tflops"] = round(2.0 * rows * (W * dl_in + rank * DH * (dd + dv) + W * DH * dv) / st["delta_products_us"] / 1e6, 2)
+        st["dense_ff_tflops"] = round(2.0 * rows * 3 * W * ff / st["dense_ff_us"] / 1e6, 2)
+        # per row and head: decay of the state, two inner products and one rank-one update over dim x vdim (fp32)
+        st["delta_scan_tflops_fp32"] = round(rows * DH * dd * dv * 7.0 / st["delta_scan_us"] / 1e6, 3)
+        if tag == "decode":
+            st["sink_attention_GBps"] = round(rows * keys * 2 * G * hd * 2 / st["sink_attention_us"] / 1e3, 1)
+            st["latent_attention_GBps"] = round(rows * keys * (2 * R + lr) * 2 / st["latent_attention_us"] / 1e3, 1)
+            st["attention_products_GBps"] = round(W * (att_in + H * hd) * 2 / st["attention_products_us"] / 1e3, 1)
+            st["dense_ff_GBps"] = round(3 * W * ff * 2 / st["dense_ff_us"] / 1e3, 1)
+            st["delta_scan_state_GBps"] = round(rows * DH * dd * dv * 4 * 2 / st["delta_scan_us"] / 1e3, 1)
+        st["layer_stack_us"] = round(b.time_stage(0, 0, 5), 2)
+    stage_times("prefill", P, P)
+    b.release(0)
+    for s_ in range(B):
+        for c0 in range(0, P, 512):
+            b.step([(s_, prompts[s_][c0:c0 + 512])], [], fetch=False)
+    toks = rng.integers(0, V, size=(steps + 8, B), dtype=np.int32)
+    for i in range(8):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+    t0 = time.perf_counter()
+    for i in range(8, 8 + steps):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+        b.step_sample()
+    dt = time.perf_counter() - t0
+    stage_times("decode", B, P)
+    out.update(value=round(B * steps / dt, 1), steps=steps, warmup=8, ms_per_step=round(dt * 1e3 / steps, 4),
+               prefill_tok_s=round(P / t_pf, 1), prefill_ms=round(t_pf * 1e3, 3),
+               prefill_tflops=round(spec.step_flops(P, P // 2) / t_pf / 1e12, 2), stages=stages, vs_baseline=None)
+    b.close()
+    eng.close()
+    out["qwen_equal_size"] = qwen_twin(Q, S, Wt, a.verelorn, W, H, G, hd, ff, V, P, B, steps, prompts, a.prefill_iters, max_ctx)
     print(json.dumps(out), flush=True)
     return 0
 

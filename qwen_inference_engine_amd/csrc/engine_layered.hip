@@ -126,7 +126,8 @@ struct LayeredBatch {
     std::vector<int64_t> conv_off;    // per layer run: the last inputs of its short convolutions (delta rule)
     std::vector<int64_t> canon_off;   // per layer run: the last normed mixer inputs (input convolution)
     float *pre = nullptr, *aux = nullptr;   // first-stage projections / convolved q, k, v; second-stage gate logits
-    int64_t m_pre = 0, m_aux = 0;
+    float* dw = nullptr;                    // delta rule in pieces: the rows' transformed queries [rows][heads * dim]
+    int64_t m_pre = 0, m_aux = 0, m_dw = 0;
     int32_t* row_k = nullptr;         // a row's index inside its entry
     float* state = nullptr;           // [slots][slot_state] fp32
     int64_t slot_state = 0;
@@ -1226,7 +1227,24 @@ static int enq_delta_scan(qie_batch* b, int r, int T, bool advance) {
     sp.state = s->state; sp.slot_stride = s->slot_state; sp.state_off = s->state_off[r];
     sp.read_state = 1; sp.write_state = advance ? 1 : 0;
     sp.out = s->olat;
-    QIE_TRY(lay::delta_scan(sp, e->stream));
+    if (s->max_count > kScanLong && s->s_loc && s->dw) {
+        // long entries: pieces from zero states side by side (end states, transition matrices, transformed
+        // queries), a carry over each entry's pieces, then the incoming states' share of every row
+        const int64_t n = (int64_t)c.heads * c.dim * c.vdim;
+        lay::DeltaScanP a = sp;
+        a.entries = s->d_chunks; a.n_entries = s->n_chunks;
+        a.state = s->s_loc; a.slot_stride = n; a.state_off = 0;
+        a.read_state = 0; a.write_state = 1;
+        a.trans = s->s_decay; a.w_out = s->dw;
+        QIE_TRY(lay::delta_scan(a, e->stream));
+        lay::DeltaCarryP k{s->d_spans, s->n_ent, c.heads, c.dim, c.vdim, s->s_loc, s->s_decay, s->s_in, s->state, s->slot_state,
+                           s->state_off[r], advance ? 1 : 0};
+        QIE_TRY(lay::delta_carry(k, e->stream));
+        lay::DeltaApplyP ap{s->d_chunks, s->n_chunks, kScanPiece, c.heads, c.dim, c.vdim, s->s_in, s->dw, s->olat};
+        QIE_TRY(lay::delta_apply(ap, e->stream));
+    } else {
+        QIE_TRY(lay::delta_scan(sp, e->stream));
+    }
     return lay::head_norm_rows(s->olat, nullptr, L.dl_norm, m->a.norm_eps, 1.0f, c.heads, c.vdim, T, s->ov, s->ov_bf, L.n_cat, 0,
                                e->stream, s->aux);
 }
@@ -1434,14 +1452,14 @@ static void lb_free(LayeredBatch* s) {
     drop_graphs(s);   // captured launches hold these buffers' addresses
     void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
                   s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf,
-                  s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf, s->pre, s->aux, s->row_k};
+                  s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf, s->pre, s->aux, s->row_k, s->dw};
     for (void* p : ps)
         if (p) hipFree(p);
     s->stack = s->x = s->proj = s->qabs = s->olat = s->ov = s->mix = s->y = s->gu = s->act = s->ffo = s->xg = s->yd = s->score =
         s->keep = nullptr;
     s->abf = s->x_bf = s->y_bf = s->ov_bf = s->act_bf = s->xg_bf = nullptr;
     s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = s->row_k = nullptr;
-    s->pre = s->aux = nullptr;
+    s->pre = s->aux = s->dw = nullptr;
     s->cap = 0;
 }
 
@@ -1507,6 +1525,7 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         A((void**)&s->stack, (m->a.depth_mix ? L + 1 : std::max<int64_t>(2, m->a.streams)) * cap * W);
         A((void**)&s->pre, cap * std::max<int64_t>(s->m_pre, 1));
         A((void**)&s->aux, cap * std::max<int64_t>(s->m_aux, 1));
+        if (s->m_dw > 0) A((void**)&s->dw, cap * s->m_dw);
         A((void**)&s->row_k, cap);
         A((void**)&s->x, cap * W);
         A((void**)&s->proj, cap * s->m_in);
@@ -1644,6 +1663,9 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
             s->m_pre = std::max<int64_t>(s->m_pre, C);
             s->m_hr = std::max<int64_t>({s->m_hr, (int64_t)c.heads * c.dim, (int64_t)c.heads * c.vdim});
             s->m_aux = std::max<int64_t>(s->m_aux, (int64_t)c.heads * c.vdim);
+            s->m_dw = std::max<int64_t>(s->m_dw, (int64_t)c.heads * c.dim);
+            s->m_state = std::max<int64_t>(s->m_state, (int64_t)c.heads * c.dim * c.vdim);
+            s->m_hd = std::max<int64_t>(s->m_hd, (int64_t)c.heads * c.dim * c.dim);
             s->m_hv = std::max<int64_t>(s->m_hv, (int64_t)c.heads * c.vdim);
             s->m_abf = std::max<int64_t>({s->m_abf, (int64_t)m->a.width, (int64_t)c.heads * c.vdim});
         } else if (d.mixer == QIE_MIXER_MINGRU) {

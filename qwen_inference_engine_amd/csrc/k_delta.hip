@@ -11,6 +11,15 @@
 // columns of one head.  q, k, g and beta of 8 rows at a time are staged in LDS (every lane of a
 // column group reads the same addresses), the next rows' values already in registers.  The state
 // is fp32 and lives with the slot; an entry that starts at position 0 starts from zero.
+//
+// Long entries run in pieces side by side.  A column s of S moves through a row as s <- A_t s + beta k v_c
+// with A_t = (I - beta k k^T) diag(g), the same A_t for every column, so over a piece s_end = M s_in + s_loc with
+// M = the product of the piece's A_t and s_loc the end state from zero.  A piece scanned from zero with dim extra
+// columns that start as the unit vectors and see v = 0 yields s_loc, M (those columns' end states) and, as those
+// columns' outputs, w_t = M_t^T q_t, M_t the product up to row t.  lay::delta_carry walks an entry's pieces
+// (s_in of the next piece = M s_in + s_loc; the slot's state = what leaves the last), lay::delta_apply adds the
+// incoming state's share s_in^T w_t to every row's output: no second scan.  Same sums as row by row up to fp32
+// rounding.
 #include "k_layered.hpp"
 
 namespace qie {
@@ -76,21 +85,23 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanP p) {
     const int4 en = p.entries[blockIdx.y];   // {first packed row, rows, slot, first position}
     const int dim = p.dim, vdim = p.vdim, G = p.G, H = p.H;
     const int gh = h / (H / G);
-    const bool colv = col < vdim;
+    // columns vdim .. vdim + dim - 1 (when p.trans): the unit vectors under v = 0, see the header
+    const bool colv = col < vdim + (p.trans ? dim : 0), idc = col >= vdim;
     const int64_t HV = (int64_t)H * vdim, HD = (int64_t)H * dim;
     float* stp = p.state + (int64_t)en.z * p.slot_stride + p.state_off + (int64_t)h * dim * vdim;
+    const bool rd = p.read_state == 2 || (p.read_state == 1 && en.w > 0);
     float S[DS_RP];
 #pragma unroll
     for (int i = 0; i < DS_RP; i++) {
         const int r = rg * DS_RP + i;
-        S[i] = (p.read_state && en.w > 0 && colv && r < dim) ? stp[(int64_t)r * vdim + col] : 0.f;
+        S[i] = idc ? (r == col - vdim ? 1.f : 0.f) : (rd && colv && r < dim) ? stp[(int64_t)r * vdim + col] : 0.f;
     }
     const int v_col = 2 * G * dim + h * vdim + col;
     for (int t0 = 0; t0 < en.y; t0 += DS_TT) {
         const int nt = min(DS_TT, en.y - t0);
         float vv[DS_TT];
 #pragma unroll
-        for (int tt = 0; tt < DS_TT; tt++) vv[tt] = (tt < nt && colv) ? p.qkv[(int64_t)(en.x + t0 + tt) * p.ld_qkv + v_col] : 0.f;
+        for (int tt = 0; tt < DS_TT; tt++) vv[tt] = (tt < nt && colv && !idc) ? p.qkv[(int64_t)(en.x + t0 + tt) * p.ld_qkv + v_col] : 0.f;
         __syncthreads();   // the previous rows have been read
         for (int i = tid; i < nt * dimP; i += 256) {
             const int tt = i / dimP, r = i % dimP;
@@ -107,20 +118,21 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanP p) {
             const float* kk = sk + tt * dimP + rg * DS_RP;
             const float* qq = sq + tt * dimP + rg * DS_RP;
             const float* gg = sg + tt * dimP + rg * DS_RP;
-            float dot = 0.f;
+            // four partial sums per inner product: the adds of one sum wait for each other
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
             for (int i = 0; i < DS_RP; i += 4) {
                 const float4 g4 = *reinterpret_cast<const float4*>(gg + i);
                 const float4 k4 = *reinterpret_cast<const float4*>(kk + i);
                 S[i] *= g4.x; S[i + 1] *= g4.y; S[i + 2] *= g4.z; S[i + 3] *= g4.w;
-                dot = fmaf(k4.x, S[i], dot);
-                dot = fmaf(k4.y, S[i + 1], dot);
-                dot = fmaf(k4.z, S[i + 2], dot);
-                dot = fmaf(k4.w, S[i + 3], dot);
+                d0 = fmaf(k4.x, S[i], d0);
+                d1 = fmaf(k4.y, S[i + 1], d1);
+                d2 = fmaf(k4.z, S[i + 2], d2);
+                d3 = fmaf(k4.w, S[i + 3], d3);
             }
-            dot = group_sum_lp<LP>(dot);
+            const float dot = group_sum_lp<LP>((d0 + d1) + (d2 + d3));
             const float u = sb[tt] * (vv[tt] - dot);
-            float o = 0.f;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int i = 0; i < DS_RP; i += 4) {
                 const float4 k4 = *reinterpret_cast<const float4*>(kk + i);
@@ -129,16 +141,31 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanP p) {
                 S[i + 1] = fmaf(k4.y, u, S[i + 1]);
                 S[i + 2] = fmaf(k4.z, u, S[i + 2]);
                 S[i + 3] = fmaf(k4.w, u, S[i + 3]);
-                o = fmaf(q4.x, S[i], o);
-                o = fmaf(q4.y, S[i + 1], o);
-                o = fmaf(q4.z, S[i + 2], o);
-                o = fmaf(q4.w, S[i + 3], o);
+                o0 = fmaf(q4.x, S[i], o0);
+                o1 = fmaf(q4.y, S[i + 1], o1);
+                o2 = fmaf(q4.z, S[i + 2], o2);
+                o3 = fmaf(q4.w, S[i + 3], o3);
             }
-            o = group_sum_lp<LP>(o);
-            if (rg == 0 && colv) p.out[(int64_t)(en.x + t0 + tt) * HV + (int64_t)h * vdim + col] = o;
+            const float o = group_sum_lp<LP>((o0 + o1) + (o2 + o3));
+            if (rg == 0 && colv) {
+                if (!idc)
+                    p.out[(int64_t)(en.x + t0 + tt) * HV + (int64_t)h * vdim + col] = o;
+                else
+                    p.w_out[(int64_t)(en.x + t0 + tt) * HD + (int64_t)h * dim + (col - vdim)] = o;
+            }
         }
     }
-    if (!colv || !p.write_state) return;
+    if (!colv) return;
+    if (idc) {   // column col - vdim of the piece's transition matrix
+        float* mt = p.trans + ((int64_t)en.z * H + h) * dim * dim + (col - vdim);
+#pragma unroll
+        for (int i = 0; i < DS_RP; i++) {
+            const int r = rg * DS_RP + i;
+            if (r < dim) mt[(int64_t)r * dim] = S[i];
+        }
+        return;
+    }
+    if (!p.write_state) return;
 #pragma unroll
     for (int i = 0; i < DS_RP; i++) {
         const int r = rg * DS_RP + i;
@@ -152,8 +179,9 @@ int delta_scan(const DeltaScanP& p, hipStream_t st) {
                 "delta_scan: %d heads over %d key heads of %d / %d (dim at most %d)", p.H, p.G, p.dim, p.vdim, 16 * DS_RP);
     int LP = 1;
     while (LP * DS_RP < p.dim) LP *= 2;
-    const int cpb = 256 / LP;
-    const dim3 grid((unsigned)p.H, (unsigned)p.n_entries, (unsigned)((p.vdim + cpb - 1) / cpb));
+    QIE_REQUIRE(!p.trans || p.w_out, "delta_scan: the transition matrices go with the rows' transformed queries");
+    const int cpb = 256 / LP, ncols = p.vdim + (p.trans ? p.dim : 0);
+    const dim3 grid((unsigned)p.H, (unsigned)p.n_entries, (unsigned)((ncols + cpb - 1) / cpb));
     const size_t shm = (size_t)(3 * DS_TT * DS_RP * LP + DS_TT) * 4;
     switch (LP) {
         case 1: hipLaunchKernelGGL(delta_scan_kernel<1>, grid, dim3(256), shm, st, p); break;
@@ -162,6 +190,96 @@ int delta_scan(const DeltaScanP& p, hipStream_t st) {
         case 8: hipLaunchKernelGGL(delta_scan_kernel<8>, grid, dim3(256), shm, st, p); break;
         default: hipLaunchKernelGGL(delta_scan_kernel<16>, grid, dim3(256), shm, st, p); break;
     }
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ pieces: carry and apply
+// One block per (entry, head, 8 state columns): the columns live in LDS, thread (r0, c) owns rows r0, r0 + 32, ...
+constexpr int DC_COLS = 8;
+
+__global__ __launch_bounds__(256) void delta_carry_kernel(DeltaCarryP p) {
+    extern __shared__ float ss[];   // [dim][DC_COLS]
+    const int4 sp = p.spans[blockIdx.x];   // {first piece, pieces, slot, first position}
+    const int h = blockIdx.y, c = threadIdx.x % DC_COLS, r0 = threadIdx.x / DC_COLS, col = blockIdx.z * DC_COLS + c;
+    const int dim = p.dim, vdim = p.vdim, H = p.H;
+    const bool colv = col < vdim;
+    float* stp = p.state + (int64_t)sp.z * p.slot_stride + p.state_off + (int64_t)h * dim * vdim;
+    for (int r = r0; r < dim; r += 32) ss[r * DC_COLS + c] = (sp.w > 0 && colv) ? stp[(int64_t)r * vdim + col] : 0.f;
+    __syncthreads();
+    for (int k = 0; k < sp.y; k++) {
+        const int64_t ph = (int64_t)(sp.x + k) * H + h;
+        float acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int r = r0 + 32 * i;
+            if (r < dim) {
+                if (colv) p.s_in[(ph * dim + r) * vdim + col] = ss[r * DC_COLS + c];
+                float a = colv ? p.s_loc[(ph * dim + r) * vdim + col] : 0.f;
+                const float* mr = p.trans + (ph * dim + r) * dim;
+                for (int j = 0; j < dim; j++) a = fmaf(mr[j], ss[j * DC_COLS + c], a);
+                acc[i] = a;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int r = r0 + 32 * i;
+            if (r < dim) ss[r * DC_COLS + c] = acc[i];
+        }
+        __syncthreads();
+    }
+    if (!p.write_state || !colv) return;
+    for (int r = r0; r < dim; r += 32) stp[(int64_t)r * vdim + col] = ss[r * DC_COLS + c];
+}
+
+int delta_carry(const DeltaCarryP& p, hipStream_t st) {
+    QIE_REQUIRE(p.spans && p.n_spans > 0 && p.s_loc && p.trans && p.s_in && p.state && p.dim > 0 && p.dim <= 512 && p.vdim > 0,
+                "delta_carry: bad arguments");
+    const dim3 grid((unsigned)p.n_spans, (unsigned)p.H, (unsigned)((p.vdim + DC_COLS - 1) / DC_COLS));
+    hipLaunchKernelGGL(delta_carry_kernel, grid, dim3(256), (size_t)p.dim * DC_COLS * 4, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// out[t, h, col] += sum_j s_in[piece][h][j][col] w[t, h, j]: one block per (piece, head, 64 columns), j in tiles of 64
+// through LDS; thread (rq, col) owns rows rq, rq + 4, ... of the piece (at most 64).
+__global__ __launch_bounds__(256) void delta_apply_kernel(DeltaApplyP p) {
+    __shared__ float sw[64 * 64];   // [row][j]
+    __shared__ float st[64 * 64];   // [j][col]
+    const int4 en = p.chunks[blockIdx.x];   // {first packed row, rows, piece index, 0}
+    const int h = blockIdx.y, lc = threadIdx.x & 63, rq = threadIdx.x >> 6, col = blockIdx.z * 64 + lc;
+    const int dim = p.dim, vdim = p.vdim, H = p.H;
+    const float* sin = p.s_in + ((int64_t)en.z * H + h) * dim * vdim;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    for (int j0 = 0; j0 < dim; j0 += 64) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+            const int a = i >> 6, bq = i & 63;   // w: row a, j bq;  state: j a, column bq
+            sw[i] = (a < en.y && j0 + bq < dim) ? p.w[(int64_t)(en.x + a) * H * dim + (int64_t)h * dim + j0 + bq] : 0.f;
+            st[i] = (j0 + a < dim && blockIdx.z * 64 + bq < vdim) ? sin[(int64_t)(j0 + a) * vdim + blockIdx.z * 64 + bq] : 0.f;
+        }
+        __syncthreads();
+        for (int jj = 0; jj < 64; jj++) {
+            const float sv = st[jj * 64 + lc];
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[i] = fmaf(sw[(rq + 4 * i) * 64 + jj], sv, acc[i]);
+        }
+    }
+    if (col >= vdim) return;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int a = rq + 4 * i;
+        if (a < en.y) p.out[(int64_t)(en.x + a) * H * vdim + (int64_t)h * vdim + col] += acc[i];
+    }
+}
+
+int delta_apply(const DeltaApplyP& p, hipStream_t st) {
+    QIE_REQUIRE(p.chunks && p.n_chunks > 0 && p.s_in && p.w && p.out && p.max_rows <= 64, "delta_apply: bad arguments (pieces of at most 64 rows)");
+    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.H, (unsigned)((p.vdim + 63) / 64));
+    hipLaunchKernelGGL(delta_apply_kernel, grid, dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();
     return 0;
 }

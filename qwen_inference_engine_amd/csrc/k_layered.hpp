@@ -370,10 +370,41 @@ struct DeltaScanP {
     int H, G, dim, vdim;
     float* state;
     int64_t slot_stride, state_off;
-    int read_state, write_state;
+    int read_state;         // 0: start from zero; 1: read the state unless the entry starts at position 0; 2: always read
+    int write_state;
     float* out;             // [T][H * vdim]
+    // pieces of long entries (entries {first packed row, rows, piece index, 0}, state = per-piece end states): with
+    // trans [pieces][H][dim][dim] the piece's transition matrix M (s_end = M s_in + s_loc) is written there and
+    // w_out [T][H * dim] receives w_t = M_t^T q_t, M_t the transition from the piece's start to row t
+    float* trans;
+    float* w_out;
 };
 int delta_scan(const DeltaScanP& p, hipStream_t st);
+// Walks every entry's pieces (spans {first piece, pieces, slot, first position}): s_in[c] = the state entering piece
+// c, from the slot's state (zero at position 0) through s <- M_c s + s_loc[c]; the slot's state = what leaves the
+// last piece (write_state).  s_loc, s_in [pieces][H][dim][vdim].
+struct DeltaCarryP {
+    const int4* spans;
+    int n_spans;
+    int H, dim, vdim;
+    const float* s_loc;
+    const float* trans;
+    float* s_in;
+    float* state;
+    int64_t slot_stride, state_off;
+    int write_state;
+};
+int delta_carry(const DeltaCarryP& p, hipStream_t st);
+// out[t, h, :] += s_in[piece of t][h]^T w[t, h, :] over the pieces {first packed row, rows (<= 64), piece index, 0}
+struct DeltaApplyP {
+    const int4* chunks;
+    int n_chunks, max_rows;
+    int H, dim, vdim;
+    const float* s_in;
+    const float* w;
+    float* out;
+};
+int delta_apply(const DeltaApplyP& p, hipStream_t st);
 // Rows of W: x = xin + (wb ? rms(v) * (w_one + wb) : v) (when v) + add (when add); then (when wn)
 // h = rms(x) * (w_one + wn) with its bf16 image.  xin may be x.  w_one = 1: weight vectors stored
 // around zero; 0: plain weights.

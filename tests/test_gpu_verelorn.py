@@ -302,6 +302,21 @@ def test_long_portions_beside_short_ones(model):
     assert rel(np.concatenate([r1[300:], r2[:7]]), wb) < m.tol
 
 
+@pytest.mark.parametrize("name", ["delta", "delta-grouped", "delta-wide-key", "delta-many-columns", "delta-huge-key"])
+def test_delta_rule_in_pieces_equals_row_by_row(model, name):
+    """Portions above 128 rows run as pieces of 64 rows side by side (transition matrices, a carry, the incoming
+    states' share); from a fresh and from a kept state, a ragged last piece, beside a short entry."""
+    m = model(ALONE[name], seed=21, max_ctx=512, tweak=slow_decay)
+    a, b = m.tokens(341), m.tokens(5)
+    wa, wb = m.ref(a), m.ref(b)
+    r1 = m.batch.step([(1, b[:3]), (0, a[:150])], range(153))
+    r2 = m.batch.step([(0, a[150:]), (1, b[3:])], range(193))
+    assert rel(np.concatenate([r1[3:], r2[:191]]), wa) < m.tol
+    assert rel(np.concatenate([r1[:3], r2[191:]]), wb) < m.tol
+    m.batch.release(0)
+    assert rel(feed(m, 0, a, [129, 2, 200]), wa) < m.tol
+
+
 def test_bf16_sizes_of_the_matrix_core_kernels(model):
     """Head sizes that are multiples of 32 and a width that is a multiple of 8: the shapes the bf16 engine's
     matrix-core products and attention kernels take."""
