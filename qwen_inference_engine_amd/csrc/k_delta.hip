@@ -207,25 +207,61 @@ __global__ __launch_bounds__(256) void delta_carry_kernel(DeltaCarryP p) {
     float* stp = p.state + (int64_t)sp.z * p.slot_stride + p.state_off + (int64_t)h * dim * vdim;
     for (int r = r0; r < dim; r += 32) ss[r * DC_COLS + c] = (sp.w > 0 && colv) ? stp[(int64_t)r * vdim + col] : 0.f;
     __syncthreads();
+    const int nr = (dim - r0 + 31) / 32;   // this thread's rows r0, r0 + 32, ... (at most 16)
     for (int k = 0; k < sp.y; k++) {
         const int64_t ph = (int64_t)(sp.x + k) * H + h;
+        const float* mt = p.trans + ph * dim * dim;
         float acc[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int r = r0 + 32 * i;
-            if (r < dim) {
-                if (colv) p.s_in[(ph * dim + r) * vdim + col] = ss[r * DC_COLS + c];
-                float a = colv ? p.s_loc[(ph * dim + r) * vdim + col] : 0.f;
-                const float* mr = p.trans + (ph * dim + r) * dim;
-                for (int j = 0; j < dim; j++) a = fmaf(mr[j], ss[j * DC_COLS + c], a);
-                acc[i] = a;
+            acc[i] = 0.f;
+            if (i < nr && colv) {
+                p.s_in[(ph * dim + r) * vdim + col] = ss[r * DC_COLS + c];
+                acc[i] = p.s_loc[(ph * dim + r) * vdim + col];
             }
+        }
+        // rows in groups of four share every read of the state column; four matrix entries per load where dim allows
+        for (int i0 = 0; i0 < nr; i0 += 4) {
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            const float* m0 = mt + (int64_t)(r0 + 32 * i0) * dim;
+            const float* m1 = m0 + (i0 + 1 < nr ? 32 * dim : 0);
+            const float* m2 = m0 + (i0 + 2 < nr ? 64 * dim : 0);
+            const float* m3 = m0 + (i0 + 3 < nr ? 96 * dim : 0);
+            int j = 0;
+            if ((dim & 3) == 0) {
+                for (; j < dim; j += 4) {
+                    const float4 x0 = *reinterpret_cast<const float4*>(m0 + j), x1 = *reinterpret_cast<const float4*>(m1 + j);
+                    const float4 x2 = *reinterpret_cast<const float4*>(m2 + j), x3 = *reinterpret_cast<const float4*>(m3 + j);
+                    const float s0 = ss[j * DC_COLS + c], s1 = ss[(j + 1) * DC_COLS + c], s2 = ss[(j + 2) * DC_COLS + c],
+                                s3 = ss[(j + 3) * DC_COLS + c];
+                    a0 = fmaf(x0.w, s3, fmaf(x0.z, s2, fmaf(x0.y, s1, fmaf(x0.x, s0, a0))));
+                    a1 = fmaf(x1.w, s3, fmaf(x1.z, s2, fmaf(x1.y, s1, fmaf(x1.x, s0, a1))));
+                    a2 = fmaf(x2.w, s3, fmaf(x2.z, s2, fmaf(x2.y, s1, fmaf(x2.x, s0, a2))));
+                    a3 = fmaf(x3.w, s3, fmaf(x3.z, s2, fmaf(x3.y, s1, fmaf(x3.x, s0, a3))));
+                }
+            }
+            for (; j < dim; j++) {
+                const float sv = ss[j * DC_COLS + c];
+                a0 = fmaf(m0[j], sv, a0);
+                a1 = fmaf(m1[j], sv, a1);
+                a2 = fmaf(m2[j], sv, a2);
+                a3 = fmaf(m3[j], sv, a3);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i += 4)
+                if (i == i0) {
+                    acc[i] += a0;
+                    acc[i + 1] += a1;
+                    acc[i + 2] += a2;
+                    acc[i + 3] += a3;
+                }
         }
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int r = r0 + 32 * i;
-            if (r < dim) ss[r * DC_COLS + c] = acc[i];
+            if (i < nr) ss[r * DC_COLS + c] = acc[i];
         }
         __syncthreads();
     }
