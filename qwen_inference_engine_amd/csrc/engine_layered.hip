@@ -1814,8 +1814,8 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
                 "qie_engine_create_layered: repeated group [%d, %d) x %d of %d layers", arch->loop_start, arch->loop_stop,
                 arch->loop_times, arch->n_layers);
     QIE_REQUIRE(!loops || arch->block == QIE_BLOCK_SANDWICH, "qie_engine_create_layered: repeated groups go with the sandwich block");
-    QIE_REQUIRE(arch->streams >= 0 && arch->streams <= 8 && arch->canon_taps >= 0 && arch->canon_taps <= 64,
-                "qie_engine_create_layered: %d residual streams (at most 8), %d input taps (at most 64)", arch->streams, arch->canon_taps);
+    QIE_REQUIRE(arch->streams >= 0 && arch->streams <= 32 && arch->canon_taps >= 0 && arch->canon_taps <= 64,
+                "qie_engine_create_layered: %d residual streams (at most 32), %d input taps (at most 64)", arch->streams, arch->canon_taps);
     QIE_REQUIRE(arch->block == QIE_BLOCK_PRENORM || (arch->streams == 0 && arch->canon_taps == 0 && !arch->embed_norm &&
                                                      arch->norm_offset == 0.f),
                 "qie_engine_create_layered: residual streams, the input convolution, the embedding norm and the norm offset "

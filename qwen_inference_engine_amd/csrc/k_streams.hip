@@ -31,14 +31,19 @@ __device__ __forceinline__ float bsum(float v, float* red) {
 
 // ------------------------------------------------------------------ hyper-connections
 // One block per row.  A thread owns coordinates w = tid, tid + 256, ... of all N rows of its token:
-// new rows from the old ones, the read-out u, u kept in LDS for the norm's second pass.
-template <int N>
-__global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p) {
+// new rows from the old ones, the read-out u, u kept in LDS for the norm's second pass.  NT: the number of rows
+// at compile time (1 .. 8), or 0 for any number up to kMaxStreams.
+constexpr int kMaxStreams = 32;
+
+template <int NT>
+__global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p, int stage) {
     extern __shared__ float su[];   // [W]
     __shared__ float red[4];
-    __shared__ float cm[N * N + 2 * N];
+    constexpr int NA = NT ? NT : kMaxStreams;
+    const int N = NT ? NT : p.n;
+    __shared__ float cm[NA * NA + 2 * NA];
     const int64_t r0 = (int64_t)blockIdx.x * p.W;
-    if (threadIdx.x < N * N) cm[threadIdx.x] = p.y ? p.mix[threadIdx.x] : 0.f;
+    for (int i = threadIdx.x; i < N * N; i += 256) cm[i] = p.y ? p.mix[i] : 0.f;
     if (threadIdx.x < N) {
         cm[N * N + threadIdx.x] = p.y ? p.out[threadIdx.x] : 0.f;
         cm[N * N + N + threadIdx.x] = p.in ? p.in[threadIdx.x] : 0.f;
@@ -46,12 +51,12 @@ __global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p) {
     __syncthreads();
     float ss = 0.f;
     for (int w = threadIdx.x; w < p.W; w += 256) {
-        float x[N];
+        float x[NA];
 #pragma unroll
         for (int s = 0; s < N; s++) x[s] = p.X[s * p.plane + r0 + w];
         if (p.y) {
             const float y = p.y[r0 + w];
-            float nx[N];
+            float nx[NA];
 #pragma unroll
             for (int t = 0; t < N; t++) {
                 float a = cm[N * N + t] * y;
@@ -75,7 +80,7 @@ __global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p) {
             float u = 0.f;
 #pragma unroll
             for (int s = 0; s < N; s++) u = fmaf(cm[N * N + N + s], x[s], u);
-            su[w] = u;
+            if (stage) su[w] = u;
             ss += u * u;
         }
     }
@@ -83,19 +88,26 @@ __global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p) {
     ss = bsum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)p.W + p.eps);
     for (int w = threadIdx.x; w < p.W; w += 256) {
-        const float o = su[w] * inv * (p.w_one + p.wn[w]);   // the thread's own LDS store above
+        float u = 0.f;
+        if (stage) {
+            u = su[w];   // the thread's own LDS store above
+        } else {         // rows wider than the staging: the read-out again from the thread's own stores, same order
+#pragma unroll
+            for (int s = 0; s < N; s++) u = fmaf(cm[N * N + N + s], p.X[s * p.plane + r0 + w], u);
+        }
+        const float o = u * inv * (p.w_one + p.wn[w]);
         p.h[r0 + w] = o;
         if (p.h_bf) p.h_bf[r0 + w] = f2bf(o);
     }
 }
 
 int stream_step(const StreamStepP& p, hipStream_t st) {
-    QIE_REQUIRE(p.n >= 1 && p.n <= 8 && p.X && p.T > 0 && p.W > 0, "stream_step: %d streams", p.n);
+    QIE_REQUIRE(p.n >= 1 && p.n <= kMaxStreams && p.X && p.T > 0 && p.W > 0, "stream_step: %d streams (at most %d)", p.n, kMaxStreams);
     QIE_REQUIRE(!p.y || (p.mix && p.out), "stream_step: an update needs its coefficients");
     QIE_REQUIRE(!p.in || (p.wn && p.h), "stream_step: a read-out needs its norm weight and a destination");
-    const size_t shm = (size_t)p.W * 4;
-    QIE_REQUIRE(shm <= 48 * 1024, "stream_step: width %d above the kernel's staging", p.W);
-#define QIE_SS(N) hipLaunchKernelGGL(stream_step_kernel<N>, dim3(p.T), dim3(256), shm, st, p)
+    const int stage = (size_t)p.W * 4 <= 48 * 1024 ? 1 : 0;
+    const size_t shm = stage ? (size_t)p.W * 4 : 0;
+#define QIE_SS(N) hipLaunchKernelGGL(stream_step_kernel<N>, dim3(p.T), dim3(256), shm, st, p, stage)
     switch (p.n) {
         case 1: QIE_SS(1); break;
         case 2: QIE_SS(2); break;
@@ -104,7 +116,8 @@ int stream_step(const StreamStepP& p, hipStream_t st) {
         case 5: QIE_SS(5); break;
         case 6: QIE_SS(6); break;
         case 7: QIE_SS(7); break;
-        default: QIE_SS(8); break;
+        case 8: QIE_SS(8); break;
+        default: QIE_SS(0); break;
     }
 #undef QIE_SS
     QIE_LAUNCH_CHECK();

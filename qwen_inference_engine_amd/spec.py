@@ -720,8 +720,8 @@ def _verelorn_from_config(cfg: dict, name: str) -> LayeredSpec:
         layers.append(LayerSpec(mixer, mlp))
     streams = int(cfg.get("streams") or 0)
     taps = int((cfg.get("canon") or {}).get("taps", 0))
-    if streams < 0 or streams > 8:
-        raise ValueError(f"streams {streams}: at most 8 residual streams")
+    if streams < 0 or streams > 32:
+        raise ValueError(f"streams {streams}: at most 32 residual streams")
     return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), depth_mix=False,
                        block="prenorm", tied_head=False, norm_offset=1.0, streams=streams, canon_taps=taps, embed_norm=True)
 

@@ -125,7 +125,7 @@ ALONE = {
 
 
 @pytest.mark.parametrize("name", sorted(ALONE))
-@pytest.mark.parametrize("streams,taps", [(3, 3), (0, 0), (1, 1), (8, 5)])
+@pytest.mark.parametrize("streams,taps", [(3, 3), (0, 0), (1, 1), (8, 5), (11, 2)])
 def test_each_mechanism_alone(model, name, streams, taps):
     m = model(ALONE[name], seed=3, streams=streams, taps=taps)
     toks = m.tokens(37)

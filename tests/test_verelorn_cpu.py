@@ -62,7 +62,7 @@ def test_refusals():
     cfg["layers"][0]["mixer"]["vdim"] = 8
     with pytest.raises(ValueError):
         S.spec_from_config(cfg)
-    cfg = public(O.config([attn()], streams=9))
+    cfg = public(O.config([attn()], streams=33))
     with pytest.raises(ValueError):
         S.spec_from_config(cfg)
 
