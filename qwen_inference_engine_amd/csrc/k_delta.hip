@@ -38,13 +38,13 @@ template <int LP> __device__ __forceinline__ float group_sum_lp(float v) {
 }
 }  // namespace
 
-// One block per row; a wave per (q or k) head, then the gates.
+// gridDim.y blocks per row (several when the step has few rows); a wave per (q or k) head, then the gates.
 __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepP p) {
     const int64_t t = blockIdx.x;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, y = blockIdx.y, ny = gridDim.y;
     float* qk = p.qkv + t * p.ld_qkv;
     const float qs = 1.0f / sqrtf((float)p.dim);
-    for (int hh = wave; hh < 2 * p.G; hh += 4) {
+    for (int hh = y * 4 + wave; hh < 2 * p.G; hh += 4 * ny) {
         float* x = qk + (int64_t)hh * p.dim;   // q heads, then k heads
         float ss = 0.f;
         for (int i = lane; i < p.dim; i += 64) ss += x[i] * x[i];
@@ -53,9 +53,10 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepP p) {
         for (int i = lane; i < p.dim; i += 64) x[i] *= inv;
     }
     float* row = p.proj + t * p.ld;
-    for (int h = threadIdx.x; h < p.H; h += 256) row[p.b_col + h] = 1.0f / (1.0f + expf(-row[p.b_col + h]));
+    if (y == 0)
+        for (int h = threadIdx.x; h < p.H; h += 256) row[p.b_col + h] = 1.0f / (1.0f + expf(-row[p.b_col + h]));
     float* a = p.a + t * (int64_t)p.H * p.dim;
-    for (int i = threadIdx.x; i < p.H * p.dim; i += 256) {
+    for (int i = y * 256 + threadIdx.x; i < p.H * p.dim; i += 256 * ny) {
         const float z = a[i] + p.dt_bias[i];
         const float sp = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
         a[i] = expf(-p.exp_a[i / p.dim] * sp);
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepP p) {
 int delta_prep(const DeltaPrepP& p, int T, hipStream_t st) {
     QIE_REQUIRE(p.qkv && p.proj && p.a && p.dt_bias && p.exp_a && p.H > 0 && p.G > 0 && p.H % p.G == 0 && p.dim > 0,
                 "delta_prep: bad arguments");
-    hipLaunchKernelGGL(delta_prep_kernel, dim3(T), dim3(256), 0, st, p);
+    const int ny = T <= 64 ? std::min(8, std::max(1, p.H * p.dim / 256)) : 1;
+    hipLaunchKernelGGL(delta_prep_kernel, dim3(T, ny), dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();
     return 0;
 }

@@ -933,7 +933,7 @@ __global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, con
                                                              int out_col, const float* gate) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int h = wave; h < heads; h += 4) {
+    for (int h = blockIdx.y * 4 + wave; h < heads; h += 4 * gridDim.y) {
         const float* x = o + (t * heads + h) * vdim;
         const float* x2 = o2 ? o2 + (t * heads + h) * vdim : nullptr;
         float ss = 0.f;
@@ -954,7 +954,8 @@ __global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, con
 }
 int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
                    uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st, const float* gate) {
-    hipLaunchKernelGGL(head_norm_rows_kernel, dim3(T), dim3(256), 0, st, o, o2, w, eps, scale, heads, vdim, out, out_bf, ld_out,
+    const int ny = T <= 64 ? std::min(8, (heads + 3) / 4) : 1;   // few rows: a row's heads over several blocks
+    hipLaunchKernelGGL(head_norm_rows_kernel, dim3(T, ny), dim3(256), 0, st, o, o2, w, eps, scale, heads, vdim, out, out_bf, ld_out,
                        out_col, gate);
     QIE_LAUNCH_CHECK();
     return 0;

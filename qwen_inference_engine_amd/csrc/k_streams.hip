@@ -41,14 +41,28 @@ __global__ __launch_bounds__(256) void stream_step_kernel(StreamStepP p, int sta
     __shared__ float red[4];
     constexpr int NA = NT ? NT : kMaxStreams;
     const int N = NT ? NT : p.n;
-    __shared__ float cm[NA * NA + 2 * NA];
     const int64_t r0 = (int64_t)blockIdx.x * p.W;
-    for (int i = threadIdx.x; i < N * N; i += 256) cm[i] = p.y ? p.mix[i] : 0.f;
-    if (threadIdx.x < N) {
-        cm[N * N + threadIdx.x] = p.y ? p.out[threadIdx.x] : 0.f;
-        cm[N * N + N + threadIdx.x] = p.in ? p.in[threadIdx.x] : 0.f;
+    // the coefficient tables: the same addresses for every lane (scalar loads, in flight beside the rows' loads);
+    // an unknown number of rows keeps them in LDS instead
+    __shared__ float cms[NT ? 1 : NA * NA + 2 * NA];
+    float cmr[NT ? NT * NT + 2 * NT : 1];
+    if (NT) {
+#pragma unroll
+        for (int i = 0; i < NT * NT; i++) cmr[i] = p.y ? p.mix[i] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NT; i++) {
+            cmr[NT * NT + i] = p.y ? p.out[i] : 0.f;
+            cmr[NT * NT + NT + i] = p.in ? p.in[i] : 0.f;
+        }
+    } else {
+        for (int i = threadIdx.x; i < N * N; i += 256) cms[i] = p.y ? p.mix[i] : 0.f;
+        if (threadIdx.x < N) {
+            cms[N * N + threadIdx.x] = p.y ? p.out[threadIdx.x] : 0.f;
+            cms[N * N + N + threadIdx.x] = p.in ? p.in[threadIdx.x] : 0.f;
+        }
+        __syncthreads();
     }
-    __syncthreads();
+    const float* cm = NT ? cmr : cms;
     float ss = 0.f;
     for (int w = threadIdx.x; w < p.W; w += 256) {
         float x[NA];
