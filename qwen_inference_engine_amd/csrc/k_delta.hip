@@ -74,15 +74,17 @@ int delta_prep(const DeltaPrepP& p, int T, hipStream_t st) {
 
 constexpr int DS_RP = 32;   // state rows per lane
 constexpr int DS_TT = 8;    // rows staged at a time
+constexpr int DS_SEG = DS_RP + 4;   // a lane group's 32 staged values, padded by 16 bytes: the LP groups of a column read
+                                    // different banks (unpadded they sit 128 bytes apart, the same banks)
 
 template <int LP>
 __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanP p) {
     extern __shared__ float sm[];
-    constexpr int dimP = DS_RP * LP, CPB = 256 / LP;
+    constexpr int dimP = DS_RP * LP, dimS = DS_SEG * LP, CPB = 256 / LP;
     float* sq = sm;
-    float* sk = sm + DS_TT * dimP;
-    float* sg = sm + 2 * DS_TT * dimP;
-    float* sb = sm + 3 * DS_TT * dimP;
+    float* sk = sm + DS_TT * dimS;
+    float* sg = sm + 2 * DS_TT * dimS;
+    float* sb = sm + 3 * DS_TT * dimS;
     const int h = blockIdx.x, tid = threadIdx.x, rg = tid % LP, col = blockIdx.z * CPB + tid / LP;
     const int4 en = p.entries[blockIdx.y];   // {first packed row, rows, slot, first position}
     const int dim = p.dim, vdim = p.vdim, G = p.G, H = p.H;
@@ -110,16 +112,17 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanP p) {
             const int64_t row = en.x + t0 + tt;
             const bool in = r < dim;
             const float* qr = p.qkv + row * p.ld_qkv;
-            sq[i] = in ? qr[gh * dim + r] : 0.f;
-            sk[i] = in ? qr[(G + gh) * dim + r] : 0.f;
-            sg[i] = in ? p.g[row * HD + (int64_t)h * dim + r] : 1.f;
+            const int d = tt * dimS + (r / DS_RP) * DS_SEG + r % DS_RP;
+            sq[d] = in ? qr[gh * dim + r] : 0.f;
+            sk[d] = in ? qr[(G + gh) * dim + r] : 0.f;
+            sg[d] = in ? p.g[row * HD + (int64_t)h * dim + r] : 1.f;
         }
         if (tid < nt) sb[tid] = p.beta[(int64_t)(en.x + t0 + tid) * p.ld_beta + h];
         __syncthreads();
         for (int tt = 0; tt < nt; tt++) {
-            const float* kk = sk + tt * dimP + rg * DS_RP;
-            const float* qq = sq + tt * dimP + rg * DS_RP;
-            const float* gg = sg + tt * dimP + rg * DS_RP;
+            const float* kk = sk + tt * dimS + rg * DS_SEG;
+            const float* qq = sq + tt * dimS + rg * DS_SEG;
+            const float* gg = sg + tt * dimS + rg * DS_SEG;
             // four partial sums per inner product: the adds of one sum wait for each other
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
@@ -184,7 +187,7 @@ int delta_scan(const DeltaScanP& p, hipStream_t st) {
     QIE_REQUIRE(!p.trans || p.w_out, "delta_scan: the transition matrices go with the rows' transformed queries");
     const int cpb = 256 / LP, ncols = p.vdim + (p.trans ? p.dim : 0);
     const dim3 grid((unsigned)p.H, (unsigned)p.n_entries, (unsigned)((ncols + cpb - 1) / cpb));
-    const size_t shm = (size_t)(3 * DS_TT * DS_RP * LP + DS_TT) * 4;
+    const size_t shm = (size_t)(3 * DS_TT * DS_SEG * LP + DS_TT) * 4;
     switch (LP) {
         case 1: hipLaunchKernelGGL(delta_scan_kernel<1>, grid, dim3(256), shm, st, p); break;
         case 2: hipLaunchKernelGGL(delta_scan_kernel<2>, grid, dim3(256), shm, st, p); break;
