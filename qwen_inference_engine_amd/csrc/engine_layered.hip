@@ -1216,8 +1216,10 @@ static int enq_delta_scan(qie_batch* b, int r, int T, bool advance) {
     cv.residual = 0; cv.silu = 1;
     cv.out = s->pre; cv.ld_out = C; cv.out_bf = nullptr;
     cv.entries = s->d_ent; cv.n_entries = s->n_ent;
-    QIE_TRY(lay::causal_conv(cv, T, e->stream));
-    if (advance) QIE_TRY(lay::causal_conv_state(cv, e->stream));
+    if (advance)
+        QIE_TRY(lay::causal_conv_advance(cv, T, e->stream));
+    else
+        QIE_TRY(lay::causal_conv(cv, T, e->stream));
     lay::DeltaPrepP pp{s->pre, C, s->proj, L.n_in, L.col_b, s->qabs, L.dl_dt_bias, L.dl_exp_a, c.heads, c.kv_heads, c.dim, c.vdim};
     QIE_TRY(lay::delta_prep(pp, T, e->stream));
     lay::DeltaScanP sp{};
@@ -1296,8 +1298,7 @@ static int enq_run_prenorm(qie_batch* b, int r, int T, bool h_ready, bool* next_
         cv.residual = 1; cv.silu = 0;
         cv.out = s->y; cv.ld_out = W; cv.out_bf = s->y_bf;
         cv.entries = s->d_ent; cv.n_entries = s->n_ent;
-        QIE_TRY(lay::causal_conv(cv, T, st));
-        QIE_TRY(lay::causal_conv_state(cv, st));
+        QIE_TRY(lay::causal_conv_advance(cv, T, st));
     }
     switch (L.d.mixer) {
         case QIE_MIXER_MINGRU: QIE_TRY(enq_mingru_mixer(b, r, T)); break;
@@ -1413,10 +1414,12 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
         float* raw = m->a.embed_norm ? s->mix : xs;
         QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, raw, nullptr, T, W, m->a.vocab, e->stream, m->a.embed_scale,
                                 m->a.pos_embed == QIE_POS_SINUSOID ? s->row_pos : nullptr, m->pos_freq));
-        if (m->a.embed_norm)
+        if (m->a.embed_norm)   // the normed rows go to every stream's plane
             QIE_TRY(lay::add_norm(raw, raw, nullptr, nullptr, nullptr, m->w_embed, xs, nullptr, T, W, m->a.norm_eps, e->stream,
-                                  m->a.norm_offset));
-        for (int k = 1; k < n; k++) QIE_HIP(hipMemcpyAsync(xs + k * plane, xs, (size_t)T * W * 4, hipMemcpyDeviceToDevice, e->stream));
+                                  m->a.norm_offset, std::max(n, 1), plane));
+        else
+            for (int k = 1; k < n; k++)
+                QIE_HIP(hipMemcpyAsync(xs + k * plane, xs, (size_t)T * W * 4, hipMemcpyDeviceToDevice, e->stream));
         bool ready = false;
         for (int r = 0; r < (int)m->runs.size(); r++) QIE_TRY(enq_run_prenorm(b, r, T, ready, &ready));
         x = n > 0 ? s->x : xs;

@@ -335,6 +335,9 @@ struct CausalConvP {
 };
 int causal_conv(const CausalConvP& p, int T, hipStream_t st);
 int causal_conv_state(const CausalConvP& p, hipStream_t st);
+// Both in order; steps of at most kConvFusedRows rows in one launch (a thread per entry and channel)
+constexpr int kConvFusedRows = 64;
+int causal_conv_advance(const CausalConvP& p, int T, hipStream_t st);
 // out[t, c] = in[t, col + c] / sqrt(mean_c in^2 + eps) * (w_one + w[c]), c < n (out may be in + col)
 int rms_rows(const float* in, int64_t ld_in, int col, int n, const float* w, float w_one, float eps, float* out, int64_t ld_out,
              uint16_t* out_bf, int T, hipStream_t st);
@@ -408,8 +411,9 @@ int delta_apply(const DeltaApplyP& p, hipStream_t st);
 // Rows of W: x = xin + (wb ? rms(v) * (w_one + wb) : v) (when v) + add (when add); then (when wn)
 // h = rms(x) * (w_one + wn) with its bf16 image.  xin may be x.  w_one = 1: weight vectors stored
 // around zero; 0: plain weights.
+// copies > 1: h is written `copies` times, `plane` elements apart (the rows of several residual streams start equal).
 int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,
-             int T, int W, float eps, hipStream_t st, float w_one = 1.0f);
+             int T, int W, float eps, hipStream_t st, float w_one = 1.0f, int copies = 1, int64_t plane = 0);
 
 // The producers below also write the bf16 image of their result when the *_bf pointer is set
 // (bf16 engines: the next product reads it; no separate rounding pass).

@@ -963,7 +963,8 @@ int head_norm_rows(const float* o, const float* o2, const float* w, float eps, f
 
 // ------------------------------------------------------------------ residual add + next norm
 __global__ __launch_bounds__(256) void add_norm_kernel(float* x, const float* xin, const float* v, const float* wb, const float* add,
-                                                       const float* wn, float* h, uint16_t* h_bf, int W, float eps, float w_one) {
+                                                       const float* wn, float* h, uint16_t* h_bf, int W, float eps, float w_one, int copies,
+                                                       int64_t plane) {
     __shared__ float red[4];
     const int64_t r0 = (int64_t)blockIdx.x * W;
     float inv_v = 0.f;
@@ -990,13 +991,14 @@ __global__ __launch_bounds__(256) void add_norm_kernel(float* x, const float* xi
     for (int i = threadIdx.x; i < W; i += 256) {
         const float o = x[r0 + i] * inv_x * (w_one + wn[i]);   // the thread's own store above
         h[r0 + i] = o;
+        for (int k = 1; k < copies; k++) h[k * plane + r0 + i] = o;
         if (h_bf) h_bf[r0 + i] = f2bf(o);
     }
 }
 int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,
-             int T, int W, float eps, hipStream_t st, float w_one) {
+             int T, int W, float eps, hipStream_t st, float w_one, int copies, int64_t plane) {
     QIE_REQUIRE(x && xin && (!wn || h), "add_norm: bad arguments");
-    hipLaunchKernelGGL(add_norm_kernel, dim3(T), dim3(256), 0, st, x, xin, v, wb, add, wn, h, h_bf, W, eps, w_one);
+    hipLaunchKernelGGL(add_norm_kernel, dim3(T), dim3(256), 0, st, x, xin, v, wb, add, wn, h, h_bf, W, eps, w_one, copies, plane);
     QIE_LAUNCH_CHECK();
     return 0;
 }

@@ -193,6 +193,51 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(CausalConvP p) {
     }
 }
 
+// Steps of few rows: one thread per (entry, channel) does both - the entry's rows in order, then the state - in one
+// launch (the thread reads the old state for its rows before it writes the new one).
+__global__ __launch_bounds__(256) void causal_conv_fused_kernel(CausalConvP p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.C) return;
+    const int4 en = p.entries[blockIdx.y];   // {first packed row, rows, slot, first position}
+    float* sb = p.state + (int64_t)en.z * p.slot_stride + p.state_off;
+    const float* w = p.w + (int64_t)c * p.taps;
+    for (int k = 0; k < en.y; k++) {
+        const int t = en.x + k, pos = en.w + k;
+        const float cur = p.in[(int64_t)t * p.ld_in + p.col + c];
+        float a = 0.f;
+        for (int j = 0; j < p.taps; j++) {
+            const int back = p.taps - 1 - j;
+            float x;
+            if (back == 0)
+                x = cur;
+            else if (back <= k)
+                x = p.in[(int64_t)(t - back) * p.ld_in + p.col + c];
+            else if (pos - back >= 0)
+                x = sb[(int64_t)(k - back + p.taps - 1) * p.C + c];
+            else
+                x = 0.f;
+            a = fmaf(w[j], x, a);
+        }
+        if (p.residual) a += cur;
+        if (p.silu) a = a / (1.0f + expf(-a));
+        const int64_t o = (int64_t)t * p.ld_out + c;
+        p.out[o] = a;
+        if (p.out_bf) p.out_bf[o] = f2bf(a);
+    }
+    const int n = p.taps - 1;
+    for (int i = 0; i < n; i++) {
+        const int q = en.y - n + i;
+        float x;
+        if (q >= 0)
+            x = p.in[(int64_t)(en.x + q) * p.ld_in + p.col + c];
+        else if (en.w + q >= 0)
+            x = sb[(int64_t)(i + en.y) * p.C + c];
+        else
+            x = 0.f;
+        sb[(int64_t)i * p.C + c] = x;
+    }
+}
+
 static int conv_check(const CausalConvP& p) {
     QIE_REQUIRE(p.in && p.w && p.C > 0 && p.taps >= 1 && p.taps <= 64, "causal_conv: %d channels, %d taps", p.C, p.taps);
     QIE_REQUIRE(p.taps == 1 || p.state, "causal_conv: the state is missing");
@@ -203,6 +248,17 @@ int causal_conv(const CausalConvP& p, int T, hipStream_t st) {
     QIE_REQUIRE(p.out && p.row_slot && p.row_pos && p.row_k, "causal_conv: bad arguments");
     const int64_t n = (int64_t)T * p.C;
     hipLaunchKernelGGL(causal_conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, T);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+int causal_conv_advance(const CausalConvP& p, int T, hipStream_t st) {
+    QIE_TRY(conv_check(p));
+    QIE_REQUIRE(p.out && p.entries && p.n_entries > 0, "causal_conv_advance: bad arguments");
+    if (T > kConvFusedRows || p.out == p.in) {
+        QIE_TRY(causal_conv(p, T, st));
+        return causal_conv_state(p, st);
+    }
+    hipLaunchKernelGGL(causal_conv_fused_kernel, dim3((unsigned)((p.C + 255) / 256), (unsigned)p.n_entries), dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();
     return 0;
 }
