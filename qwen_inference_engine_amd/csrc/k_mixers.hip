@@ -342,6 +342,21 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
     const int64_t o0 = (int64_t)row * a.ld_out + a.out_col + (int64_t)hh * vdim;
     const float* cs = a.rot_values ? a.vrope_cos + (int64_t)qpos * (vdim / 2) : nullptr;
     const float* sn = a.rot_values ? a.vrope_sin + (int64_t)qpos * (vdim / 2) : nullptr;
+    // the gates of all of the column's coordinates first: a load placed between the stores below would wait for
+    // them (the two arrays may overlap as far as the compiler knows)
+    const bool gated = a.gate_col >= 0 && a.gate_elem;
+    float gf[DV][4];
+    if (gated) {
+        const float* gp = a.proj + (int64_t)row * a.ld + a.gate_col + hh * vdim + 4 * g;
+#pragma unroll
+        for (int dv = 0; dv < DV; dv++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) gf[dv][j] = gp[16 * dv + j];
+#pragma unroll
+        for (int dv = 0; dv < DV; dv++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) gf[dv][j] = 1.0f / (1.0f + __expf(-gf[dv][j]));
+    }
 #pragma unroll
     for (int dv = 0; dv < DV; dv++) {
         float o[4];
@@ -372,7 +387,7 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             float y = o[j] * a.out_scale;
-            if (a.gate_col >= 0 && a.gate_elem) y *= 1.0f / (1.0f + __expf(-a.proj[(int64_t)row * a.ld + a.gate_col + hh * vdim + v0 + j]));
+            if (gated) y *= gf[dv][j];
             a.out[o0 + v0 + j] = y;
             if (a.out_bf) a.out_bf[o0 + v0 + j] = f2bf(y);
         }
@@ -611,28 +626,31 @@ __global__ __launch_bounds__(256) void gqa_attn_combine_kernel(GqaAttnMfmaP P, i
     gf32x4_t acc[DV];
 #pragma unroll
     for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
-    // two parts a turn, every load of the turn issued before its first use; a part that saw no key
-    // of the column has l = 0 and zero sums
-    for (int z0 = 0; z0 < P.S; z0 += 2) {
-        const int z1 = min(z0 + 1, P.S - 1);
-        const float w0 = ml[32 * z0 + 1] == 0.f ? 0.f : __expf(ml[32 * z0] - M);
-        const float w1 = (z0 + 1 >= P.S || ml[32 * z1 + 1] == 0.f) ? 0.f : __expf(ml[32 * z1] - M);
-        L += ml[32 * z0 + 1] * w0 + ml[32 * z1 + 1] * w1;
-        const float* p0 = P.part_o + ((u0 + z0) * 16 + n) * vdim + 4 * g;
-        const float* p1 = P.part_o + ((u0 + z1) * 16 + n) * vdim + 4 * g;
-        float4 o0[DV], o1[DV];
+    // several parts a turn (a turn is one trip to memory), every load of the turn issued before its first use; a
+    // part that saw no key of the column has l = 0 and zero sums
+    constexpr int PT = DV <= 8 ? 4 : 2;
+    for (int z0 = 0; z0 < P.S; z0 += PT) {
+        float w[PT];
+        float4 o[PT][DV];
 #pragma unroll
-        for (int dv = 0; dv < DV; dv++) {
-            o0[dv] = *reinterpret_cast<const float4*>(p0 + 16 * dv);
-            o1[dv] = *reinterpret_cast<const float4*>(p1 + 16 * dv);
+        for (int k = 0; k < PT; k++) {
+            const int zk = min(z0 + k, P.S - 1);
+            const float l = ml[32 * zk + 1];
+            w[k] = (z0 + k >= P.S || l == 0.f) ? 0.f : __expf(ml[32 * zk] - M);
+            L += l * w[k];
+            const float* pk = P.part_o + ((u0 + zk) * 16 + n) * vdim + 4 * g;
+#pragma unroll
+            for (int dv = 0; dv < DV; dv++) o[k][dv] = *reinterpret_cast<const float4*>(pk + 16 * dv);
         }
 #pragma unroll
-        for (int dv = 0; dv < DV; dv++) {
-            acc[dv][0] += o0[dv].x * w0 + o1[dv].x * w1;
-            acc[dv][1] += o0[dv].y * w0 + o1[dv].y * w1;
-            acc[dv][2] += o0[dv].z * w0 + o1[dv].z * w1;
-            acc[dv][3] += o0[dv].w * w0 + o1[dv].w * w1;
-        }
+        for (int k = 0; k < PT; k++)
+#pragma unroll
+            for (int dv = 0; dv < DV; dv++) {
+                acc[dv][0] += o[k][dv].x * w[k];
+                acc[dv][1] += o[k][dv].y * w[k];
+                acc[dv][2] += o[k][dv].z * w[k];
+                acc[dv][3] += o[k][dv].w * w[k];
+            }
     }
     gqa_store<DV>(a, acc, gqa_out_factor(a, L, M, grp.x + tI, hh), grp.x + tI, hh, pos0 + tI, g);
 }
