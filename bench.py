@@ -480,11 +480,11 @@ def verelorn_model(S, size):
     W, H, G, hd, rot, LH, ld, lr, lv, R, QR, DH, DG, dd, dv, taps_d, rank, ff, streams, taps, V = VERELORN_SIZES[size]
     mlp = {"kind": "dense", "ff": ff}
     lat = lambda kv_from: {"type": "latent_attention", "mlp": mlp, "mixer": dict(
-        {"heads": LH, "dim": ld, "rot_dim": lr, "vdim": lv, "kv_rank": R, "q_rank": QR, "rot": {"base": 1e6, "dims": lr},
+        {"heads": LH, "dim": ld, "rot_dim": lr, "vdim": lv, "kv_rank": R, "q_rank": QR, "rot": {"base": 10000.0, "dims": lr},
          "scale": (ld + lr) ** -0.5}, **({} if kv_from is None else {"kv_from": kv_from}))}
     att = {"type": "attention", "mlp": mlp, "mixer": {
         "heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
-        "rot": {"base": 250000.0, "dims": rot, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 1024}}}}
+        "rot": {"base": 500000.0, "dims": rot, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
     dlt = {"type": "channel_delta", "mlp": None, "mixer": {"heads": DH, "kv_heads": DG, "dim": dd, "vdim": dv, "conv": taps_d}}
     cfg = {"architecture": "Verelorn", "layers": [lat(None), att, dlt, lat(0)], "norm": {"eps": 1e-5}, "streams": streams,
            "canon": {"taps": taps}, "vocab": V, "width": W}

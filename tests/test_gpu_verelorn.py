@@ -262,7 +262,7 @@ def sharp(T, cfg):
 @pytest.mark.parametrize("page_tokens", [16, 64])
 def test_far_keys_and_page_borders_with_sharp_softmax(model, page_tokens):
     m = model([attn(heads=4, kv_heads=2, dim=16, rot_dims=8, base=100.0), latent(base=100.0), latent(kv_from=1, base=100.0)],
-              seed=9, tweak=sharp, page_tokens=page_tokens, max_ctx=448)
+              seed=9, tweak=sharp, page_tokens=page_tokens, max_ctx=512)
     toks = m.tokens(330)
     want = m.ref(toks)
     moved = m.ref([(t + 1) % m.vocab for t in toks[:16]] + toks[16:])
