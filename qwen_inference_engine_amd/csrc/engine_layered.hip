@@ -4,7 +4,8 @@
 // A layered engine is a qie_engine whose `lm` holds the architecture and the device weights; a
 // batch of it is a paged qie_batch whose pool holds, per layer run, the rows its mixer caches
 // (latent rows, or K and V rows of a grouped-query attention), whose `lb` holds the step's
-// activations and, for recurrent mixers, one fp32 state per slot and layer run.  Slots, the block table and the page pool are the
+// activations and, for recurrent mixers and convolutions over time, one fp32 state per slot and layer run (recurrent
+// states, the convolutions' last inputs).  Slots, the block table and the page pool are the
 // batch's own (ensure_pages / drop_pages / flush_table, qie_batch_release, qie_batch_page_stats).
 //
 // A step packs the rows of all entries (portions of prompts and single tokens alike) end to

@@ -5,8 +5,10 @@
 //   lay::gqa_attention   grouped-query softmax attention over the paged rows with a causal,
 //                        sliding or block-local mask and an optional log-distance bias; the
 //                        weighted sum of turned values is turned back
-//                        and / or a linear one with a slope per head; softmax weights, or sigmoid
-//                        weights with a bias per head; an optional sigmoid gate per head
+//                        and / or a linear one with a slope per head; softmax weights (optionally with a
+//                        sink: one more term exp(sink_h) in the denominator, no key, no value), or sigmoid
+//                        weights with a bias per head; an optional sigmoid gate per head or per coordinate;
+//                        bias vectors on q and k (gqa_post)
 //   lay::gated_scan      gated linear recurrence with an fp32 state per slot and head
 //   lay::mingru_scan     minGRU: a recurrence per channel, update gate and candidate from the current input alone
 //   lay::head_norm_rows  per-head RMS norm with a weight
